@@ -1,4 +1,5 @@
 from .base import ConfigReader, architecture_name, read_config_json
+from .dafidra import DafidraConfig
 from .llama import LlamaConfig, RopeScaling
 
-__all__ = ["ConfigReader", "architecture_name", "read_config_json", "LlamaConfig", "RopeScaling"]
+__all__ = ["ConfigReader", "architecture_name", "read_config_json", "LlamaConfig", "RopeScaling", "DafidraConfig"]

@@ -105,7 +105,10 @@ def read_config_json(model_dir: str) -> dict:
 
 
 def architecture_name(raw: Mapping[str, Any], where: str = "config.json") -> str:
+    """The registry key: ``architectures[0]``, or, in folders that name one, ``architecture``."""
+    if isinstance(raw.get("architecture"), str) and "architectures" not in raw:
+        return raw["architecture"]
     archs = raw.get("architectures")
     if not isinstance(archs, (list, tuple)) or not archs or not isinstance(archs[0], str):
-        raise ConfigError(f"{where}: 'architectures' must be a non-empty list of names")
+        raise ConfigError(f"{where}: 'architectures' must be a non-empty list of names (or 'architecture' a name)")
     return archs[0]

@@ -1,4 +1,4 @@
-// Causal attention over the paged cache for any head size (multiple of 16, up to 256),
+// Causal attention over the paged cache for any head size up to 256,
 // any number of heads and groups, both storage types, prompts and single tokens alike.
 // One wave per (token, head); scores, softmax and the weighted sum are float32.
 //
@@ -8,6 +8,13 @@
 // with lo = 0, or p - window + 1 when a window is given.  Causality is the loop bound.
 // The softmax is exact: no constant is added to the denominator (the reference's paged
 // kernel adds 1e-6, src/ops/kernels/cuda/paged_attention.cu:71).
+//
+// Options, each off when its pointer is null (or vd == hd):
+//   * values of another width than keys (vd features per head; pages [page, kv head, vd, slot]);
+//   * a distance bias: slope[head] * (p - t) is taken off the scaled score of key t;
+//   * a sink per head: exp(sink[head]) joins the denominator once; it has no key and no value,
+//     is not scaled and gets no bias;
+//   * an output gate: head h's output at token t is multiplied by gate[t, h] (float32).
 //
 // Keys are visited 64 at a time with the usual running maximum / running sum, so the
 // result for a token depends only on that token's position and its request's pages.
@@ -25,7 +32,8 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     T* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ req_of_token, const int* __restrict__ positions, int nh, int nkv, int hd, int page_size,
-    float scale, int window, long num_pages, float* __restrict__ part) {
+    float scale, int window, long num_pages, float* __restrict__ part, int vd, const float* __restrict__ slopes,
+    const float* __restrict__ sinks, const float* __restrict__ gate) {
   __shared__ float qs[PI_MAX_HEAD_DIM];
   __shared__ float ps[PI_WAVE];
   __shared__ long voff[PI_WAVE];   // values are stored [page, kv_head, head_dim, slot]
@@ -40,6 +48,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
   const int* bt = block_table + (long)req_of_token[t] * table_width;
   float m = -INFINITY, l = 0.f;
   float acc[PI_MAX_HEAD_DIM / PI_WAVE] = {0.f, 0.f, 0.f, 0.f};
+  const float slope = slopes ? slopes[h] : 0.f;
   __syncthreads();
   // this wave's keys: all of lo..p, or the z-th of gridDim.z ranges of whole 64-key groups
   const int splits = gridDim.z;
@@ -57,18 +66,23 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
       const long page = blk < table_width ? bt[blk] : -1;
       if (page >= 0 && page < num_pages) {
         off = ((page * nkv + g) * page_size + (key % page_size)) * hd;
-        vo = (page * nkv + g) * (long)page_size * hd + (key % page_size);
+        vo = (page * nkv + g) * (long)page_size * vd + (key % page_size);
         const T* kr = k_cache + off;
         float dot = 0.f;
-        for (int d = 0; d < hd; d += 4) {          // in ascending order of d, four features per load
-          float kv[4];
-          load4(kr + d, kv);
-          dot = fmaf(qs[d], kv[0], dot);
-          dot = fmaf(qs[d + 1], kv[1], dot);
-          dot = fmaf(qs[d + 2], kv[2], dot);
-          dot = fmaf(qs[d + 3], kv[3], dot);
+        if ((hd & 3) == 0) {
+          for (int d = 0; d < hd; d += 4) {        // in ascending order of d, four features per load
+            float kv[4];
+            load4(kr + d, kv);
+            dot = fmaf(qs[d], kv[0], dot);
+            dot = fmaf(qs[d + 1], kv[1], dot);
+            dot = fmaf(qs[d + 2], kv[2], dot);
+            dot = fmaf(qs[d + 3], kv[3], dot);
+          }
+        } else {                                   // a head size that is no multiple of four: one feature per load
+          for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
         }
         s = dot * scale;
+        if (slopes) s -= slope * (float)(p - key);
       } else {
         s = __builtin_nanf("");  // a key without a page: make it visible, never read outside the pool
       }
@@ -95,7 +109,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
 #pragma unroll
           for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
             const int d = lane + i * PI_WAVE;
-            if (d < hd) {
+            if (d < vd) {
               float vv[4];
               load4(vr + (long)d * page_size, vv);
               acc[i] = fmaf(p0, vv[0], acc[i]);
@@ -109,7 +123,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
 #pragma unroll
           for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
             const int d = lane + i * PI_WAVE;
-            if (d < hd) acc[i] = fmaf(pk, to_float(vr[(long)d * page_size]), acc[i]);
+            if (d < vd) acc[i] = fmaf(pk, to_float(vr[(long)d * page_size]), acc[i]);
           }
         }
       }
@@ -120,24 +134,32 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
   }
   if (splits > 1) {
     // [token, head, range, hd + 2]: the un-normalised sum, then the range's maximum and sum of weights
-    float* mine = part + (((long)t * nh + h) * splits + blockIdx.z) * (hd + 2);
+    float* mine = part + (((long)t * nh + h) * splits + blockIdx.z) * (vd + 2);
 #pragma unroll
     for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
       const int d = lane + i * PI_WAVE;
-      if (d < hd) mine[d] = acc[i];
+      if (d < vd) mine[d] = acc[i];
     }
     if (lane == 0) {
-      mine[hd] = m;
-      mine[hd + 1] = l;
+      mine[vd] = m;
+      mine[vd + 1] = l;
     }
     return;
   }
-  T* o = out + t * out_stride + (long)h * hd;
-  const float inv = 1.0f / l;
+  if (sinks) {       // the sink joins the denominator once, against the common maximum
+    const float sk = sinks[h];
+    const float m_all = fmaxf(m, sk);
+    const float corr = expf(m - m_all);
+    l = l * corr + expf(sk - m_all);
+#pragma unroll
+    for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) acc[i] *= corr;
+  }
+  T* o = out + t * out_stride + (long)h * vd;
+  const float inv = (gate ? gate[t * nh + h] : 1.0f) / l;
 #pragma unroll
   for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
     const int d = lane + i * PI_WAVE;
-    if (d < hd) o[d] = from_float<T>(acc[i] * inv);
+    if (d < vd) o[d] = from_float<T>(acc[i] * inv);
   }
 }
 
@@ -145,13 +167,14 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
 // an empty range (m_s = -inf, l_s = 0) counts nothing.
 template <typename T>
 __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ part,
-                                                                   int nh, int hd, int splits) {
+                                                                   int nh, int hd, int splits, const float* __restrict__ sinks,
+                                                                   const float* __restrict__ gate) {
   const long t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* base = part + ((long)t * nh + h) * splits * (hd + 2);
-  float m = -INFINITY;
+  float m = sinks ? sinks[h] : -INFINITY;
   for (int s = 0; s < splits; ++s) m = fmaxf(m, base[s * (hd + 2) + hd]);
-  float l = 0.f;
+  float l = sinks ? expf(sinks[h] - m) : 0.f;
   float acc[PI_MAX_HEAD_DIM / PI_WAVE] = {0.f, 0.f, 0.f, 0.f};
   for (int s = 0; s < splits; ++s) {
     const float ms = base[s * (hd + 2) + hd];
@@ -164,7 +187,7 @@ __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict
     }
   }
   T* o = out + t * out_stride + (long)h * hd;
-  const float inv = 1.0f / l;
+  const float inv = (gate ? gate[t * nh + h] : 1.0f) / l;
 #pragma unroll
   for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
     const int d = lane + i * PI_WAVE;
@@ -188,31 +211,34 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
                                           const void* v_cache, int dtype, const int* block_table, int table_width,
                                           const int* req_of_token, const int* positions, int T, int nh, int nkv, int hd,
                                           int page_size, float scale, int window, long num_pages, int splits, void* part,
-                                          long part_elems, hipStream_t stream) {
+                                          long part_elems, int vd, const float* slopes, const float* sinks, const float* gate,
+                                          hipStream_t stream) {
   PI_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention: heads %d must be a positive multiple of kv heads %d", nh, nkv);
-  PI_REQUIRE(hd > 0 && hd % 16 == 0 && hd <= PI_MAX_HEAD_DIM, "attention: head_dim %d must be a multiple of 16 up to %d", hd, PI_MAX_HEAD_DIM);
+  PI_REQUIRE(hd > 0 && hd <= PI_MAX_HEAD_DIM, "attention: head_dim %d must be at most %d", hd, PI_MAX_HEAD_DIM);
   PI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "attention: bad cache geometry page_size=%d table_width=%d pages=%ld", page_size, table_width, num_pages);
   PI_REQUIRE(nh <= 65535, "attention: too many heads (%d)", nh);
   PI_REQUIRE(window >= 0, "attention: window must be >= 0, got %d", window);
   PI_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of key ranges %d", splits);
-  PI_REQUIRE(splits == 1 || (part && part_elems >= (long)T * nh * splits * (hd + 2)), "attention: workspace too small for %d key ranges", splits);
+  if (vd <= 0) vd = hd;
+  PI_REQUIRE(vd <= PI_MAX_HEAD_DIM, "attention: value width %d must be at most %d", vd, PI_MAX_HEAD_DIM);
+  PI_REQUIRE(splits == 1 || (part && part_elems >= (long)T * nh * splits * (vd + 2)), "attention: workspace too small for %d key ranges", splits);
   if (T == 0) return 0;
   const dim3 grid(T, nh, splits), block(PI_WAVE);
   if (dtype == PI_F32)
     hipLaunchKernelGGL(paged_attention_general_kernel<float>, grid, block, 0, stream, (float*)out, out_stride, (const float*)q,
                        q_stride, (const float*)k_cache, (const float*)v_cache, block_table, table_width, req_of_token,
-                       positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part);
+                       positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(paged_attention_general_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, out_stride,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width,
-                       req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part);
+                       req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate);
   else
     return pi_fail("attention: unsupported dtype %d", dtype);
   if (pi_check_launch("paged_attention_general")) return -1;
   if (splits == 1) return 0;
   if (dtype == PI_F32)
-    hipLaunchKernelGGL(merge_key_ranges_kernel<float>, dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, hd, splits);
+    hipLaunchKernelGGL(merge_key_ranges_kernel<float>, dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate);
   else
-    hipLaunchKernelGGL(merge_key_ranges_kernel<bf16_t>, dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, hd, splits);
+    hipLaunchKernelGGL(merge_key_ranges_kernel<bf16_t>, dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate);
   return pi_check_launch("merge_key_ranges");
 }

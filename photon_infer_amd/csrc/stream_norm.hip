@@ -1,0 +1,153 @@
+// Kernels around a residual stream whose sublayers are normalised on the way OUT:
+//   x <- x + mult * norm(y; w),   y = a                               (one branch)
+//                                 y = (norm(a; wa) + norm(b; wb)) / 2 (two branches side by side)
+// with norm(v; w) = v / sqrt(mean(v^2) + eps) * w.  One block per token row does the branch
+// norms, their mean, the outer norm, the scaled add into the float32 stream and, when asked,
+// the copy of the new stream in the activation type that the next sublayer's products read.
+// Sums of squares, roots and the stream are float32 throughout.  Weights are float32 (a weight
+// stored around zero is handed over as 1 + w).
+#include "common.h"
+
+template <typename TH>
+__global__ __launch_bounds__(256) void branch_norm_add_kernel(float* __restrict__ x, TH* __restrict__ h, const float* __restrict__ a,
+                                                              const float* __restrict__ wa, const float* __restrict__ b,
+                                                              const float* __restrict__ wb, const float* __restrict__ wo,
+                                                              float eps, float mult, int D) {
+  extern __shared__ float y[];          // D floats
+  __shared__ float scratch[16];
+  const long row = blockIdx.x;
+  const float* ar = a + row * D;
+  const float* br = b ? b + row * D : nullptr;
+  float sa = 0.f, sb = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float va = ar[d];
+    sa = fmaf(va, va, sa);
+    if (br) {
+      const float vb = br[d];
+      sb = fmaf(vb, vb, sb);
+    }
+  }
+  float sy = 0.f;
+  if (wa) {
+    const float ra = 1.0f / sqrtf(block_sum(sa, scratch) / D + eps);
+    const float rb = br ? 1.0f / sqrtf(block_sum(sb, scratch) / D + eps) : 0.f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+      float v = ar[d] * ra * wa[d];
+      if (br) v = 0.5f * (v + br[d] * rb * wb[d]);
+      y[d] = v;
+      sy = fmaf(v, v, sy);
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += blockDim.x) y[d] = ar[d];
+    sy = sa;
+  }
+  const float ry = 1.0f / sqrtf(block_sum(sy, scratch) / D + eps);
+  float* xr = x + row * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float v = xr[d] + mult * (y[d] * ry * wo[d]);
+    xr[d] = v;
+    if (h) h[row * D + d] = from_float<TH>(v);
+  }
+}
+
+// x (float32 stream) += mult * norm(...); h (optional, h_dtype) = the new stream.
+// wa == null: a is taken as it is (one branch, no inner norm); b == null: one branch.
+extern "C" int pi_branch_norm_add(float* x, void* h, int h_dtype, const float* a, const float* wa, const float* b,
+                                  const float* wb, const float* wo, float eps, float mult, int T, int D, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && D > 0 && D <= 40000, "branch norm: bad sizes T=%d D=%d", T, D);
+  PI_REQUIRE(x && a && wo, "branch norm: the stream, a branch and the outer weight are needed");
+  PI_REQUIRE(!b || (wa && wb), "branch norm: two branches need both their weights");
+  if (T == 0) return 0;
+  const size_t lds = (size_t)D * sizeof(float);
+  if (h && h_dtype == PI_BF16)
+    hipLaunchKernelGGL(branch_norm_add_kernel<bf16_t>, dim3(T), dim3(256), lds, stream, x, (bf16_t*)h, a, wa, b, wb, wo, eps, mult, D);
+  else if (!h || h_dtype == PI_F32)
+    hipLaunchKernelGGL(branch_norm_add_kernel<float>, dim3(T), dim3(256), lds, stream, x, (float*)h, a, wa, b, wb, wo, eps, mult, D);
+  else
+    return pi_fail("branch norm: unsupported activation dtype %d", h_dtype);
+  return pi_check_launch("branch_norm_add");
+}
+
+template <typename TO>
+__global__ void cast_stream_kernel(TO* __restrict__ out, const float* __restrict__ x, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_float<TO>(x[i]);
+}
+
+// out = the float32 stream in the activation type (for sublayers that read the stream itself)
+extern "C" int pi_cast_stream(void* out, int out_dtype, const float* x, long n, hipStream_t stream) {
+  PI_REQUIRE(n >= 0 && out_dtype == PI_BF16, "cast: only float32 -> bfloat16 is a copy worth making (dtype %d)", out_dtype);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(cast_stream_kernel<bf16_t>, dim3(ceil_div(n, 256)), dim3(256), 0, stream, (bf16_t*)out, x, n);
+  return pi_check_launch("cast_stream");
+}
+
+// ---------------------------------------------------------------- queries and keys normalised whole, then into the cache
+// One block per token.  The projection row (float32) holds [q: nh*hd | k: nkv*hd | v: nkv*vd | gate: ng].
+//   q <- q / sqrt(mean over ALL nh*hd entries + eps) * wq, times the token's temperature
+//        1 + coef * ln(floor((p + 1) / every) + 1)           (coef 0: none)
+//   k <- k / sqrt(mean over all nkv*hd entries + eps) * wk   -> key pages [page, kv head, slot, hd]
+//   v                                                         -> value pages [page, kv head, vd, slot]
+//   gate <- 1 / (1 + exp(-gate))                              -> float32 [T, ng]
+// wq / wk null: no norm of that projection.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
+    T* __restrict__ q_out, long q_stride, float* __restrict__ gate_out, const float* __restrict__ proj, long proj_stride,
+    const float* __restrict__ wq, const float* __restrict__ wk, const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    float eps, float temp_coef, int temp_every, int nh, int nkv, int hd, int vd, int ng, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages) {
+  __shared__ float scratch[16];
+  const long t = blockIdx.x;
+  const float* row = proj + t * proj_stride;
+  const int QN = nh * hd, KN = nkv * hd, VN = nkv * vd;
+  const int p = positions[t];
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < QN; i += blockDim.x) sq = fmaf(row[i], row[i], sq);
+  for (int i = threadIdx.x; i < KN; i += blockDim.x) sk = fmaf(row[QN + i], row[QN + i], sk);
+  const float rq = wq ? 1.0f / sqrtf(block_sum(sq, scratch) / QN + eps) : 1.0f;
+  const float rk = wk ? 1.0f / sqrtf(block_sum(sk, scratch) / KN + eps) : 1.0f;
+  const float temp = temp_coef != 0.f ? 1.0f + temp_coef * logf((float)((p + 1) / temp_every) + 1.0f) : 1.0f;
+  T* qr = q_out + t * q_stride;
+  for (int i = threadIdx.x; i < QN; i += blockDim.x) {
+    float v = row[i];
+    if (wq) v = v * rq * wq[i];
+    qr[i] = from_float<T>(v * temp);
+  }
+  for (int i = threadIdx.x; i < ng; i += blockDim.x) gate_out[t * ng + i] = 1.0f / (1.0f + expf(-row[QN + KN + VN + i]));
+  if (!k_cache) return;
+  const int blk = p / page_size, slot = p % page_size;
+  const long page = blk < table_width ? block_table[(long)req_of_token[t] * table_width + blk] : -1;
+  if (page < 0 || page >= num_pages) return;      // no page for this position: nothing is written
+  for (int i = threadIdx.x; i < KN; i += blockDim.x) {
+    float v = row[QN + i];
+    if (wk) v = v * rk * wk[i];
+    const int g = i / hd, d = i % hd;
+    k_cache[((page * nkv + g) * page_size + slot) * hd + d] = from_float<T>(v);
+  }
+  for (int i = threadIdx.x; i < VN; i += blockDim.x) {
+    const int g = i / vd, d = i % vd;
+    v_cache[((page * nkv + g) * vd + d) * page_size + slot] = from_float<T>(row[QN + KN + i]);
+  }
+}
+
+extern "C" int pi_qk_norm_kv_write(void* q_out, long q_stride, float* gate_out, int dtype, const float* proj, long proj_stride,
+                                   const float* wq, const float* wk, const int* positions, const int* req_of_token, float eps,
+                                   float temp_coef, int temp_every, int T, int nh, int nkv, int hd, int vd, int ng,
+                                   void* k_cache, void* v_cache, const int* block_table, int table_width, int page_size,
+                                   long num_pages, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && ng >= 0, "qk norm: bad sizes");
+  PI_REQUIRE(proj_stride >= (long)nh * hd + (long)nkv * (hd + vd) + ng, "qk norm: projection rows of %ld hold no q, k, v and gates", proj_stride);
+  PI_REQUIRE(temp_coef == 0.f || temp_every > 0, "qk norm: the temperature's period must be positive, got %d", temp_every);
+  PI_REQUIRE(!k_cache || (v_cache && block_table && req_of_token && table_width > 0 && page_size > 0 && num_pages > 0),
+             "qk norm: bad cache geometry");
+  PI_REQUIRE(ng == 0 || gate_out, "qk norm: gates without a place for them");
+  if (T == 0) return 0;
+#define QKN_GO(TT) hipLaunchKernelGGL(qk_norm_kv_write_kernel<TT>, dim3(T), dim3(256), 0, stream, (TT*)q_out, q_stride, gate_out, proj, \
+                                      proj_stride, wq, wk, positions, req_of_token, eps, temp_coef, temp_every, nh, nkv, hd, vd, ng,  \
+                                      (TT*)k_cache, (TT*)v_cache, block_table, table_width, page_size, num_pages)
+  if (dtype == PI_F32) QKN_GO(float);
+  else if (dtype == PI_BF16) QKN_GO(bf16_t);
+  else return pi_fail("qk norm: unsupported dtype %d", dtype);
+#undef QKN_GO
+  return pi_check_launch("qk_norm_kv_write");
+}

@@ -26,7 +26,7 @@ from ..errors import PhotonError
 from .options import EngineOptions
 from .step import ModelRunner, StepEntry
 
-MAX_LIVE_REQUESTS = 8        # a trace holds up to four; some room to spare
+MAX_LIVE_REQUESTS = 4        # a trace holds up to four live requests: their slots are used again
 TOKEN_ROUNDING = 64          # --max-tokens counts each request rounded up to this
 
 

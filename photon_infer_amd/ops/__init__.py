@@ -88,6 +88,14 @@ def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> N
         raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 16 up to {MAX_HEAD_DIM}")
 
 
+def check_general_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int) -> None:
+    """Sizes the general attention kernel takes (the only one for heads with options)."""
+    if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
+        raise KernelError(f"attention: {num_heads} heads is not a positive multiple of {num_kv_heads} kv heads")
+    if not (0 < head_dim <= MAX_HEAD_DIM and 0 < value_dim <= MAX_HEAD_DIM):
+        raise KernelError(f"attention: head sizes {head_dim} / {value_dim} must be at most {MAX_HEAD_DIM}")
+
+
 # ----------------------------------------------------------------------------- ops
 def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
     """out[t, :] = float32(table[ids[t], :])."""
@@ -235,11 +243,12 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool =
               _dt(w), ldw, M, N, K, int(accumulate), _stream())
 
 
-def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int, page_size: int, dtype) -> int:
-    """Keys [pages, kv_heads, page, head_dim]; values transposed, [pages, kv_heads, head_dim, page]."""
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int, page_size: int, dtype, vd: Optional[int] = None) -> int:
+    """Keys [pages, kv_heads, page, head_dim]; values transposed, [pages, kv_heads, value width (= head_dim unless given), page]."""
+    vd = hd if vd is None else vd
     if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (nkv, page_size, hd)
-            or tuple(v_cache.shape) != (k_cache.shape[0], nkv, hd, page_size)):
-        raise KernelError(f"cache: expected keys [pages, {nkv}, {page_size}, {hd}] and values [pages, {nkv}, {hd}, {page_size}], "
+            or tuple(v_cache.shape) != (k_cache.shape[0], nkv, vd, page_size)):
+        raise KernelError(f"cache: expected keys [pages, {nkv}, {page_size}, {hd}] and values [pages, {nkv}, {vd}, {page_size}], "
                           f"got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
     if k_cache.dtype != dtype or v_cache.dtype != dtype or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise KernelError(f"cache: must be contiguous {dtype}, got {k_cache.dtype}")
@@ -377,28 +386,48 @@ def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_he
                                                  block_table, page_size, scale, window, pages, write_kv, ws, leave_ranges)
 
 
+def _f32_vector(t: Optional[torch.Tensor], n: int, what: str) -> None:
+    if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n or not t.is_cuda):
+        raise KernelError(f"{what}: expected contiguous float32 with {n} entries on the GPU, got {t.dtype} {tuple(t.shape)}")
+
+
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, ctx, num_heads: int, num_kv_heads: int, head_dim: int,
-                    page_size: int, scale: float, window: int = 0, ws: Optional[KernelWorkspace] = None) -> None:
+                    page_size: int, scale: float, window: int = 0, ws: Optional[KernelWorkspace] = None, *,
+                    value_dim: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
+                    sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
     """Causal attention of every token of the step over its request's pages.
 
     ``ctx`` carries ``positions`` and ``req_of_token`` ([T] int32), the step's shape on the host
     (``q_lens``, ``kv_lens``, ``all_decode``) and, in ``plans``, the work lists that the
     matrix-core kernels want (made here when the step function has not).
+
+    Options: ``value_dim`` (values of another width than keys; ``out`` is then [T, heads * value_dim]),
+    ``slopes`` (float32 [heads]: slope * distance is taken off a key's scaled score), ``sinks``
+    (float32 [heads]: exp(sink) joins the softmax's denominator once), ``gate`` (float32
+    [T, heads]: multiplies a head's output).
     """
     _gpu(out, q, k_cache, v_cache, block_table, ctx.positions, ctx.req_of_token)
     T = q.shape[0]
-    check_attention_sizes(num_heads, num_kv_heads, head_dim)
-    if q.shape[1] != num_heads * head_dim or out.shape != (T, num_heads * head_dim) or out.dtype != q.dtype:
-        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not match {num_heads} x {head_dim}")
-    pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype)
+    vd = head_dim if value_dim is None else int(value_dim)
+    plain = vd == head_dim and slopes is None and sinks is None and gate is None
+    if plain:
+        check_attention_sizes(num_heads, num_kv_heads, head_dim)
+    else:
+        check_general_attention_sizes(num_heads, num_kv_heads, head_dim, vd)
+        _f32_vector(slopes, num_heads, "attention slopes")
+        _f32_vector(sinks, num_heads, "attention sinks")
+        _f32_vector(gate, T * num_heads, "attention gate")
+    if q.shape[1] != num_heads * head_dim or out.shape != (T, num_heads * vd) or out.dtype != q.dtype:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not match {num_heads} x {head_dim} (values {vd})")
+    pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype, vd)
     _i32(ctx.positions, "positions", T)
     _i32(ctx.req_of_token, "req_of_token", T)
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
         raise KernelError("attention: block table must be contiguous int32 [requests, width]")
     if T == 0:
         return
-    if _FAST and q.dtype == torch.bfloat16:
+    if _FAST and q.dtype == torch.bfloat16 and plain:
         from . import fast
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
                                 page_size, scale, window, pages, ws):
@@ -406,12 +435,12 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     # a step of few tokens over long contexts: its keys cut into ranges, merged by a second kernel
     # (as many as the context-length bucket asks for, so that a step gives the same bits eagerly and replayed)
     ranges = general_attention_ranges(T, num_heads, int(ctx.max_kv_len))
-    part = torch.empty(T * num_heads * ranges * (head_dim + 2), dtype=torch.float32, device=q.device) if ranges > 1 else None
+    part = torch.empty(T * num_heads * ranges * (vd + 2), dtype=torch.float32, device=q.device) if ranges > 1 else None
     _lib.call("core", "pi_paged_attention_general", out.data_ptr(), _rows(out, "attention out"), q.data_ptr(),
               _rows(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), _dt(q), block_table.data_ptr(),
               block_table.shape[1], ctx.req_of_token.data_ptr(), ctx.positions.data_ptr(), T, num_heads,
               num_kv_heads, head_dim, page_size, float(scale), int(window), pages, ranges, _ptr(part),
-              0 if part is None else part.numel(), _stream())
+              0 if part is None else part.numel(), vd, _ptr(slopes), _ptr(sinks), _ptr(gate), _stream())
 
 
 def general_attention_ranges(tokens: int, num_heads: int, max_kv_len: int) -> int:
@@ -466,3 +495,200 @@ def upload_arrays(arrays, device):
     """int32 host arrays by name -> device views of one packed copy."""
     from . import fast
     return fast.upload_arrays(arrays, device)
+
+
+# ----------------------------------------------------------------------------- streams normalised on the way out
+def cast_stream(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 stream in the activation type (itself when that is float32)."""
+    _gpu(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("cast: the stream must be contiguous float32")
+    if dtype == torch.float32:
+        return x
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _lib.call("core", "pi_cast_stream", out.data_ptr(), _dt(out), x.data_ptr(), x.numel(), _stream())
+    return out
+
+
+def branch_norm_add(x: torch.Tensor, a: torch.Tensor, w_outer: torch.Tensor, eps: float, mult: float,
+                    w_a: Optional[torch.Tensor] = None, b: Optional[torch.Tensor] = None, w_b: Optional[torch.Tensor] = None,
+                    h_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """x += mult * norm(y; w_outer) with y = a, or norm(a; w_a), or the mean of norm(a; w_a) and
+    norm(b; w_b); norm(v; w) = v / sqrt(mean(v^2) + eps) * w, all float32.  With ``h_dtype`` the new
+    stream is also returned in that type (the stream itself for float32)."""
+    _gpu(x, a, b, w_outer, w_a, w_b)
+    T, D = x.shape
+    for t, what in ((x, "stream"), (a, "branch"), (b, "second branch")):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (T, D)):
+            raise KernelError(f"branch norm: the {what} must be contiguous float32 [{T}, {D}]")
+    for t, what in ((w_outer, "outer weight"), (w_a, "branch weight"), (w_b, "second branch weight")):
+        _f32_vector(t, D, f"branch norm {what}")
+    h = None
+    if h_dtype is not None and h_dtype != torch.float32:
+        h = torch.empty((T, D), dtype=h_dtype, device=x.device)
+    _lib.call("core", "pi_branch_norm_add", x.data_ptr(), _ptr(h), _dt(h) if h is not None else PI_F32, a.data_ptr(), _ptr(w_a),
+              _ptr(b), _ptr(w_b), w_outer.data_ptr(), float(eps), float(mult), T, D, _stream())
+    if h_dtype is None:
+        return None
+    return x if h is None else h
+
+
+def qk_norm_kv_write(q_out: torch.Tensor, gate_out: Optional[torch.Tensor], proj: torch.Tensor, w_q: Optional[torch.Tensor],
+                     w_k: Optional[torch.Tensor], ctx, eps: float, temp_coef: float, temp_every: int, num_heads: int,
+                     num_kv_heads: int, head_dim: int, value_dim: int, num_gates: int, k_cache: Optional[torch.Tensor],
+                     v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor], page_size: int) -> None:
+    """From float32 projection rows [q | k | v | gates]: queries and keys each normalised over their
+    WHOLE row (all heads at once; weights float32, None: no norm), queries times the position's
+    temperature 1 + coef * ln(floor((p + 1) / every) + 1), keys and values into their pages,
+    gates through a sigmoid into ``gate_out`` (float32 [T, num_gates])."""
+    _gpu(q_out, gate_out, proj, w_q, w_k, k_cache, v_cache, block_table)
+    T = q_out.shape[0]
+    QN, KN, VN = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * value_dim
+    if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < QN + KN + VN + num_gates:
+        raise KernelError(f"qk norm: projection must be float32 [{T}, >= {QN + KN + VN + num_gates}], got {proj.dtype} {tuple(proj.shape)}")
+    if q_out.shape[1] != QN:
+        raise KernelError(f"qk norm: q has {q_out.shape[1]} columns, expected {QN}")
+    _f32_vector(w_q, QN, "qk norm query weight")
+    _f32_vector(w_k, KN, "qk norm key weight")
+    if num_gates and (gate_out is None or gate_out.dtype != torch.float32 or not gate_out.is_contiguous() or gate_out.numel() != T * num_gates):
+        raise KernelError(f"qk norm: gates need contiguous float32 [{T}, {num_gates}]")
+    pages = 0
+    if k_cache is not None:
+        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q_out.dtype, value_dim)
+        if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
+            raise KernelError("qk norm: block table must be contiguous int32 [requests, width]")
+    _i32(ctx.positions, "positions", T)
+    _i32(ctx.req_of_token, "req_of_token", T)
+    _lib.call("core", "pi_qk_norm_kv_write", q_out.data_ptr(), _rows(q_out, "q"), _ptr(gate_out), _dt(q_out), proj.data_ptr(),
+              _rows(proj, "projection"), _ptr(w_q), _ptr(w_k), ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), float(eps),
+              float(temp_coef), int(temp_every), T, num_heads, num_kv_heads, head_dim, value_dim, num_gates, _ptr(k_cache),
+              _ptr(v_cache), _ptr(block_table), block_table.shape[1] if k_cache is not None else 0, page_size, pages, _stream())
+
+
+# ----------------------------------------------------------------------------- matrix memory
+MATRIX_MEMORY_COLUMNS = 16     # value columns per wave of the scan; n and m are kept once per such group
+
+
+def matrix_memory_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
+    """Floats of one request's state: S [heads, d, dv], then (n, m) [heads, slices, d + 1]."""
+    slices = -(-value_dim // MATRIX_MEMORY_COLUMNS)
+    return heads * key_dim * value_dim + heads * slices * (key_dim + 1)
+
+
+def matrix_memory_scan(out: torch.Tensor, proj: torch.Tensor, offsets, i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float,
+                       q_scale: float, ctx, state: torch.Tensor, heads: int, key_dim: int, value_dim: int) -> None:
+    """The matrix-memory recurrence over the step's tokens, request by request, from and into the
+    requests' state rows (``state`` float32 [slots, floats], rows ``ctx.slots``).  ``proj`` float32
+    rows hold q, k, v and the two gates' pre-activations at column ``offsets`` = (q, k, v, i, f);
+    ``out`` float32 [T, heads * value_dim] gets the cell's output before its head norm."""
+    _gpu(out, proj, i_bias, f_bias, state)
+    T = out.shape[0]
+    if out.dtype != torch.float32 or not out.is_contiguous() or out.shape[1] != heads * value_dim:
+        raise KernelError(f"matrix memory: output must be contiguous float32 [{T}, {heads * value_dim}]")
+    need = max(offsets[0] + heads * key_dim, offsets[1] + heads * key_dim, offsets[2] + heads * value_dim, offsets[3] + heads, offsets[4] + heads)
+    if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < need:
+        raise KernelError(f"matrix memory: projection must be float32 [{T}, >= {need}], got {proj.dtype} {tuple(proj.shape)}")
+    _f32_vector(i_bias, heads, "matrix memory input-gate bias")
+    _f32_vector(f_bias, heads, "matrix memory forget-gate bias")
+    floats = matrix_memory_state_floats(heads, key_dim, value_dim)
+    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or state.shape[1] < floats:
+        raise KernelError(f"matrix memory: state must be contiguous float32 [slots, >= {floats}], got {state.dtype} {tuple(state.shape)}")
+    _i32(ctx.q_start, "q_start", ctx.R + 1)
+    _i32(ctx.slots, "slots", ctx.R)
+    _lib.call("core", "pi_matrix_memory_scan", out.data_ptr(), _rows(out, "out"), proj.data_ptr(), _rows(proj, "projection"),
+              int(offsets[0]), int(offsets[1]), int(offsets[2]), int(offsets[3]), int(offsets[4]), i_bias.data_ptr(),
+              f_bias.data_ptr(), float(cap), float(q_scale), ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R,
+              state.data_ptr(), state.shape[1], state.shape[0], heads, key_dim, value_dim, _stream())
+
+
+def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, value_dim: int) -> None:
+    """y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gates[t, h, :])."""
+    _gpu(y, o, gates, weight)
+    T, N = y.shape[0], heads * value_dim
+    if tuple(y.shape) != (T, N) or not y.is_contiguous():
+        raise KernelError(f"head norm: output must be contiguous [{T}, {N}]")
+    for t, what in ((o, "input"), (gates, "gates")):
+        if t.dtype != torch.float32 or t.dim() != 2 or t.shape[0] != T or t.shape[1] < N:
+            raise KernelError(f"head norm: {what} must be float32 [{T}, >= {N}]")
+    _f32_vector(weight, N, "head norm weight")
+    _lib.call("core", "pi_head_norm_gate", y.data_ptr(), _dt(y), o.data_ptr(), _rows(o, "o"), gates.data_ptr(), _rows(gates, "gates"),
+              weight.data_ptr(), float(eps), T, heads, value_dim, _stream())
+
+
+# ----------------------------------------------------------------------------- routed experts
+def route(logits: torch.Tensor, top: int, groups: int = 1, keep: int = 1, renorm: bool = False):
+    """Choose ``top`` experts per row of float32 router logits: (ids int32 [T, top], weights float32
+    [T, top]).  Scores are the softmax over all experts; with ``groups`` > 1 only experts of the
+    ``keep`` groups with the largest best score may be chosen; weights are the chosen scores
+    (divided by their sum when ``renorm``)."""
+    _gpu(logits)
+    T, E = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("routing: logits must be float32")
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _lib.call("core", "pi_route", ids.data_ptr(), weights.data_ptr(), logits.data_ptr(), _rows(logits, "router logits"), T, E,
+              int(top), int(groups), int(keep), int(bool(renorm)), _stream())
+    return ids, weights
+
+
+class ExpertRows:
+    """A step's (token, choice) entries in expert order, and the tiles of the grouped products."""
+
+    def __init__(self, row_entry, entry_row, tile_expert, tile_row0, tile_rows, top):
+        self.row_entry, self.entry_row = row_entry, entry_row
+        self.tile_expert, self.tile_row0, self.tile_rows, self.top = tile_expert, tile_row0, tile_rows, top
+
+    @property
+    def rows(self) -> int:
+        return self.row_entry.numel()
+
+
+def group_entries(ids: torch.Tensor, num_experts: int) -> ExpertRows:
+    """Sort the entries of ``ids`` (int32 [T, top]) by expert, on the device."""
+    _gpu(ids)
+    _i32(ids, "expert ids")
+    N = ids.numel()
+    tile = int(_lib.load("core").pi_group_tile_rows())
+    max_tiles = -(-N // tile) + num_experts
+    meta = torch.empty(2 * N + 3 * max_tiles, dtype=torch.int32, device=ids.device)
+    row_entry, entry_row = meta[:N], meta[N:2 * N]
+    te, t0, tr = (meta[2 * N + i * max_tiles: 2 * N + (i + 1) * max_tiles] for i in range(3))
+    _lib.call("core", "pi_group_entries", ids.data_ptr(), N, int(num_experts), row_entry.data_ptr(), entry_row.data_ptr(),
+              te.data_ptr(), t0.data_ptr(), tr.data_ptr(), max_tiles, _stream())
+    return ExpertRows(row_entry, entry_row, te, t0, tr, ids.shape[1])
+
+
+def gather_rows(src: torch.Tensor, rows: ExpertRows) -> torch.Tensor:
+    """The tokens' activations copied into expert order: [entries, D]."""
+    _gpu(src)
+    if src.dim() != 2 or not src.is_contiguous():
+        raise KernelError("gather: activations must be contiguous 2-D")
+    out = torch.empty((rows.rows, src.shape[1]), dtype=src.dtype, device=src.device)
+    _lib.call("core", "pi_gather_rows", out.data_ptr(), src.data_ptr(), _dt(src), rows.row_entry.data_ptr(), rows.rows, rows.top,
+              src.shape[1], _stream())
+    return out
+
+
+def grouped_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, rows: ExpertRows) -> None:
+    """out[row] = a[row] @ w[expert of row]^T for rows in expert order; ``w`` is [experts, N, K]."""
+    _gpu(out, a, w)
+    if w.dim() != 3 or not w.is_contiguous() or a.shape != (rows.rows, w.shape[2]) or out.shape != (rows.rows, w.shape[1]):
+        raise KernelError(f"grouped product: shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    if a.dtype != w.dtype:
+        raise KernelError(f"grouped product: activations {a.dtype} and weights {w.dtype} must have one type")
+    _lib.call("core", "pi_grouped_gemm_general", out.data_ptr(), _dt(out), _rows(out, "out"), a.data_ptr(), _dt(a), _rows(a, "a"),
+              w.data_ptr(), _dt(w), w.shape[2], w.shape[1] * w.shape[2], rows.tile_expert.data_ptr(), rows.tile_row0.data_ptr(),
+              rows.tile_rows.data_ptr(), rows.tile_expert.numel(), w.shape[1], w.shape[2], _stream())
+
+
+def combine_choices(out: torch.Tensor, y: torch.Tensor, weights: torch.Tensor, rows: ExpertRows, accumulate: bool = False) -> None:
+    """out[t] (+)= sum over the token's choices of weight * y[row of (t, choice)], in choice order (float32)."""
+    _gpu(out, y, weights)
+    T, D = out.shape
+    if out.dtype != torch.float32 or y.dtype != torch.float32 or not (out.is_contiguous() and y.is_contiguous()) or y.shape != (rows.rows, D):
+        raise KernelError(f"combine: expected float32 out [{T}, {D}] and y [{rows.rows}, {D}]")
+    if weights.dtype != torch.float32 or not weights.is_contiguous() or weights.numel() != rows.rows:
+        raise KernelError("combine: one float32 weight per entry is needed")
+    _lib.call("core", "pi_combine_choices", out.data_ptr(), y.data_ptr(), weights.data_ptr(), rows.entry_row.data_ptr(), T, rows.top, D,
+              int(bool(accumulate)), _stream())

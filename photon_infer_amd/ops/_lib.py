@@ -20,7 +20,17 @@ _SIGNATURES = {
         "pi_swiglu": [P, P, I, I, I, I, P],
         "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, P],
         "pi_gemm_general": [P, I, L, P, I, L, P, I, L, I, I, I, I, P],
-        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
+        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, P],
+        "pi_branch_norm_add": [P, P, I, P, P, P, P, P, F, F, I, I, P],
+        "pi_cast_stream": [P, I, P, L, P],
+        "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P],
+        "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, P],
+        "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, P],
+        "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
+        "pi_group_entries": [P, I, I, P, P, P, P, P, I, P],
+        "pi_gather_rows": [P, P, I, P, I, I, I, P],
+        "pi_grouped_gemm_general": [P, I, L, P, I, L, P, I, L, L, P, P, P, I, I, I, P],
+        "pi_combine_choices": [P, P, P, P, I, I, I, I, P],
         "pi_paged_attention_general_ranges": [I, I, I],
         "pi_rope_table": [P, P, P, I, I, P],
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],

@@ -5,8 +5,11 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Blo
 from .norm import RMSNorm
 from .rope import RotaryEmbedding, rope_frequencies
 from .attention import PagedAttention
+from .sink_attention import SinkWindowAttention
+from .matrix_memory import MatrixMemory
 from .mlp import SwiGLU
-from .block import PreNormBlock
+from .routed_experts import RoutedExperts
+from .block import OutputNormBlock, PreNormBlock
 from .embedding import LMHead, TokenEmbedding
 from .model import CachePlan, DecoderModel, ModelSpec, RunEntry, plan_cache
 
@@ -14,6 +17,6 @@ __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block", "FeedForward",
     "KVCacheSpec", "LayerCache", "Mixer", "Norm", "PAGE", "PagedCacheSpec", "PagedTensor", "Part", "PositionEncoding", "StateSpec",
     "StepContext", "RMSNorm", "RotaryEmbedding", "rope_frequencies", "PagedAttention", "SwiGLU",
-    "PreNormBlock", "LMHead", "TokenEmbedding", "CachePlan", "DecoderModel", "ModelSpec",
+    "PreNormBlock", "OutputNormBlock", "SinkWindowAttention", "MatrixMemory", "RoutedExperts", "LMHead", "TokenEmbedding", "CachePlan", "DecoderModel", "ModelSpec",
     "RunEntry", "plan_cache",
 ]

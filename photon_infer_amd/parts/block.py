@@ -11,6 +11,7 @@ from typing import Dict, List, Tuple
 import torch
 
 from .. import ops
+from ..errors import UnsupportedModelError
 from ..weights.loader import TensorSpec
 from .base import BLOCKS, Block, FeedForward, LayerCache, Mixer, Norm, Part, StepContext
 
@@ -54,3 +55,84 @@ class PreNormBlock(Block):
 
 
 BLOCKS.register("prenorm", PreNormBlock)
+
+
+class OutputNormBlock(Block):
+    """Sublayers that read the stream itself and are normalised on the way out:
+
+        x <- x + mult * norm1(mix(x));   x <- x + mult * norm2(ffn(x))   (no feed-forward: the first only)
+
+    ``mix`` is one mixer, or two side by side that read the same input: then each result is first
+    normalised with a weight of its own and the two are averaged.  The norms, the mean, the scaled
+    add and the copy of the new stream in the activation type are one kernel per sublayer.  The
+    mixers and the feed-forward write their result (``accumulate=False``) instead of adding it.
+
+    ``branches``: [(prefix, mixer, (prefix, norm) or None)]; ``norm1`` / ``norm2`` / ``ffn``: (prefix, part).
+    """
+
+    reads_deferred = False
+    _STREAM = "stream in the activation type"     # key in ctx.scratch: (stream, its copy) left for the next reader
+
+    def __init__(self, branches, norm1: Tuple[str, Norm], mult: float, norm2=None, ffn=None):
+        if not 1 <= len(branches) <= 2:
+            raise UnsupportedModelError(f"an output-norm block holds one mixer or two side by side, not {len(branches)}")
+        if len(branches) == 2 and any(b[2] is None for b in branches):
+            raise UnsupportedModelError("two mixers side by side each need the norm of their result")
+        if (ffn is None) != (norm2 is None):
+            raise UnsupportedModelError("a feed-forward and its norm come together")
+        self.branches = list(branches)
+        self.norm1, self.norm2, self.ffn = norm1[1], norm2[1] if norm2 else None, ffn[1] if ffn else None
+        self.mult = float(mult)
+        self._named: List[Tuple[str, Part]] = [(p, m) for p, m, _ in branches] + [n for _, _, n in branches if n is not None] + [norm1]
+        if ffn is not None:
+            self._named += [norm2, ffn]
+        for _, part in self._named:
+            if getattr(part, "accumulate", False):
+                raise UnsupportedModelError(f"{type(part).__name__} must be built with accumulate=False inside an output-norm block")
+
+    def mixers(self) -> List[Mixer]:
+        return [m for _, m, _ in self.branches]
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s.with_prefix(p) for p, part in self._named for s in part.tensor_specs()]
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        # a part's tensors: those named by its own list (prefixes here may be prefixes of one another)
+        for prefix, part in self._named:
+            names = [prefix + s.name for s in part.tensor_specs()]
+            part.load({n[len(prefix):]: tensors[n] for n in names}, dtype, device)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self._named)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for _, part in self._named for w in part.streamed_weights()]
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> None:
+        left = ctx.scratch.pop(self._STREAM, None)
+        h = left[1] if left is not None and left[0] is x else ops.cast_stream(x, self.dtype)
+        caches = cache if isinstance(cache, (list, tuple)) else [cache]
+        ctx.may_defer = False
+        outs = []
+        for (_, mixer, _), c in zip(self.branches, caches):
+            out = torch.empty_like(x)
+            mixer.forward(h, out, ctx, c)
+            outs.append(out)
+        norms = [n[1] if n is not None else None for _, _, n in self.branches]
+        eps = self.norm1.eps
+        if len(outs) == 2:
+            h = ops.branch_norm_add(x, outs[0], self.norm1.weight_f32(), eps, self.mult, norms[0].weight_f32(), outs[1],
+                                    norms[1].weight_f32(), h_dtype=self.dtype)
+        else:
+            h = ops.branch_norm_add(x, outs[0], self.norm1.weight_f32(), eps, self.mult,
+                                    norms[0].weight_f32() if norms[0] is not None else None, h_dtype=self.dtype)
+        if self.ffn is not None:
+            out = torch.empty_like(x)
+            self.ffn.forward(h, out, ctx)
+            h = ops.branch_norm_add(x, out, self.norm2.weight_f32(), self.norm2.eps, self.mult, h_dtype=self.dtype)
+        ctx.scratch[self._STREAM] = (x, h)
+
+
+BLOCKS.register("output_norm", OutputNormBlock)

@@ -19,17 +19,18 @@ from .base import Part
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, tensor_name: str = "weight"):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
+        self.tensor_name = tensor_name          # after the part's prefix; may be empty
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec("weight", (self.vocab_size, self.hidden_size), "table")]
+        return [TensorSpec(self.tensor_name, (self.vocab_size, self.hidden_size), "table")]
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.tensor_name]
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         """int32 [T] -> float32 residual stream [T, hidden]."""
@@ -41,18 +42,19 @@ class TokenEmbedding(Part):
 class LMHead(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool, tensor_name: str = "weight"):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
         self.tied = bool(tied)
+        self.tensor_name = tensor_name          # after the part's prefix; may be empty
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [] if self.tied else [TensorSpec("weight", (self.vocab_size, self.hidden_size))]
+        return [] if self.tied else [TensorSpec(self.tensor_name, (self.vocab_size, self.hidden_size))]
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device, tied_weight: Optional[torch.Tensor] = None) -> None:
         super().load(tensors, dtype, device)
-        self.weight = tied_weight if self.tied else tensors["weight"]
+        self.weight = tied_weight if self.tied else tensors[self.tensor_name]
 
     def streamed_weights(self) -> List[torch.Tensor]:
         return [self.weight]

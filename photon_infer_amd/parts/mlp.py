@@ -22,23 +22,29 @@ INTERLEAVE = 16   # rows of a matrix-core tile
 class SwiGLU(FeedForward):
     graph_safe = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"), accumulate: bool = True):
+        """``names``: the gate, up and down matrices' names after the part's prefix.
+        ``accumulate`` False: ``forward`` writes its result into the tensor it is given instead of
+        adding to it (for arrangements that normalise a sublayer's result before the residual add)."""
         if activation != "silu":
             raise UnsupportedModelError(f"gated feed-forward activation '{activation}' is not supported")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.names = tuple(names)
+        self.accumulate = bool(accumulate)
 
     def tensor_specs(self) -> List[TensorSpec]:
         I, D = self.intermediate_size, self.hidden_size
         return [
-            TensorSpec("gate_proj.weight", (I, D)),
-            TensorSpec("up_proj.weight", (I, D)),
-            TensorSpec("down_proj.weight", (D, I)),
+            TensorSpec(self.names[0], (I, D)),
+            TensorSpec(self.names[1], (I, D)),
+            TensorSpec(self.names[2], (D, I)),
         ]
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        g, u = tensors[self.names[0]], tensors[self.names[1]]
         common = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
         g, u = g.to(common), u.to(common)
         I = self.intermediate_size
@@ -52,7 +58,7 @@ class SwiGLU(FeedForward):
         else:
             self.interleave = 0                      # rows [gate | up]
             self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        self.w_down = tensors[self.names[2]]
 
     def streamed_weights(self) -> List[torch.Tensor]:
         return [self.w_gate_up, self.w_down]
@@ -61,7 +67,8 @@ class SwiGLU(FeedForward):
         act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
         ws = ctx.workspace if ctx is not None else None
         ops.gemm_swiglu(act, h, self.w_gate_up, self.interleave, ws=ws)
-        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
+        ops.gemm(x, act, self.w_down, accumulate=self.accumulate,
+                 may_defer=self.accumulate and getattr(ctx, "may_defer", False), ws=ws)
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)

@@ -2,7 +2,7 @@
 
 Formula (include/photon/ops/kernels/rmsnorm_kernel.hpp:55-87): mean of squares over
 the row, ``rms = sqrt(mean + eps)`` with eps inside the root, ``y = w * (x / rms)``;
-no mean-centring, no bias.  Sum, root and scaling run in float32; the result is
+no mean-centring, no bias.  A model that stores its weights around zero uses ``offset + w``.  Sum, root and scaling run in float32; the result is
 rounded once to the compute dtype.
 """
 from __future__ import annotations
@@ -20,17 +20,30 @@ class RMSNorm(Norm):
     consumes_deferred = True   # reads the stream through ops.rmsnorm, which adds a pending update
     graph_safe = True
 
-    def __init__(self, dim: int, eps: float):
+    def __init__(self, dim: int, eps: float, offset: float = 0.0, tensor_name: str = "weight"):
+        """``offset``: what is added to the stored weight (1.0 for weights stored around zero, used
+        as 1 + w); the sum is made and kept in float32.  ``tensor_name``: the weight's name
+        after the part's prefix (may be empty: the prefix is the name)."""
         self.dim = int(dim)
         self.eps = float(eps)
+        self.offset = float(offset)
+        self.tensor_name = tensor_name
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec("weight", (self.dim,), "norm")]
+        return [TensorSpec(self.tensor_name, (self.dim,), "norm_zero" if self.offset else "norm")]
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.tensor_name]
+        if self.offset:
+            self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
+
+    def weight_f32(self) -> torch.Tensor:
+        """The weight as the kernels that want float32 weights take it (made once)."""
+        if getattr(self, "_w32", None) is None:
+            self._w32 = self.weight.to(torch.float32).contiguous()
+        return self._w32
 
     def forward(self, x: torch.Tensor, ctx=None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         m = x.shape[0] if rows is None else rows.shape[0]

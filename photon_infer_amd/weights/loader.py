@@ -28,8 +28,8 @@ class TensorSpec:
     """One tensor a part expects.
 
     ``role`` drives random initialisation only: "matrix" and "table" are drawn from
-    N(0, std), "norm" follows the norm rule (ones or U(0.5, 1.5)), "int_table" holds
-    integers.
+    N(0, std), "norm" follows the norm rule (ones or U(0.5, 1.5)), "norm_zero" the same
+    around zero (zeros or U(-0.5, 0.5)), "bias" is N(0, 1), "int_table" holds integers.
     """
 
     name: str

@@ -36,6 +36,10 @@ def random_tensors(specs: Iterable[TensorSpec], seed: int, std: float = 0.02, no
         g = _generator(seed, s.name)
         if s.role == "norm":
             t = torch.ones(s.shape) if norm_init == "ones" else torch.rand(s.shape, generator=g) + 0.5
+        elif s.role == "norm_zero":      # weights stored around zero and used as offset + w
+            t = torch.zeros(s.shape) if norm_init == "ones" else torch.rand(s.shape, generator=g) - 0.5
+        elif s.role == "bias":           # per-head numbers of order one (gate biases, sinks)
+            t = torch.randn(s.shape, generator=g, dtype=torch.float32)
         elif s.role == "int_table":
             out[s.name] = torch.randint(0, 2**15, s.shape, generator=g, dtype=torch.int32)
             continue
