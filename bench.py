@@ -1,7 +1,7 @@
 #!/usr/bin/python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra]
                     [--batch 8,1,64] [--context 4096] [--dtype bf16|fp32]
 
 Every workload prints ONE JSON line.  The default, ``decode1b`` (Llama 3.2 1B layer sizes):  ``value`` is decoded tokens per second at batch 8 with the context
@@ -35,6 +35,11 @@ waited for the GPU.  After demo/compare_batching_methods.cpp:251-309 of the refe
 ``--workload mixed8b`` (Llama 3.1 8B layer sizes): steps that hold one 512-token portion of a
 prompt late in a context of 8,192 beside 64 decoding requests at that context: milliseconds per
 mixed step, and the step's flops and bytes against the peaks.
+
+``--workload dafidra``: the Dafidra design (windowed sink attention beside a matrix memory, dense and
+routed feed-forwards) at layer sizes like Llama 3.2 1B's and 3B's, beside a Llama of the same width,
+depth and vocabulary: a 2,048-token prompt and decode steps at batch 8, both through the same step
+functions.  ``value`` is Dafidra's decoded tokens per second at the first size.
 
 Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
 """
@@ -77,7 +82,7 @@ def make_runner(cfg_raw, layers, dtype, max_batch, max_cache_tokens, seed=0, max
     from photon_infer_amd.engine import EngineOptions, ModelRunner
     from photon_infer_amd.registry import build_model_spec, config_from_dict
 
-    raw = dict(cfg_raw, num_hidden_layers=layers)
+    raw = dict(cfg_raw, num_hidden_layers=layers) if "layers" not in cfg_raw else dict(cfg_raw, layers=list(cfg_raw["layers"])[:layers])
     cfg = config_from_dict(raw)
     spec = build_model_spec(cfg)
     tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
@@ -86,6 +91,8 @@ def make_runner(cfg_raw, layers, dtype, max_batch, max_cache_tokens, seed=0, max
     for s in spec.tensor_specs():
         if s.role == "norm":
             tensors[s.name] = torch.ones(s.shape, dtype=tdtype, device="cuda")
+        elif s.role == "norm_zero":       # weights used as 1 + w
+            tensors[s.name] = torch.zeros(s.shape, dtype=tdtype, device="cuda")
         else:
             tensors[s.name] = (torch.randn(s.shape, generator=gen, device="cuda", dtype=torch.float32) * 0.02).to(tdtype)
     opts = EngineOptions(dtype="bfloat16" if dtype == "bf16" else "float32", block_size=BLOCK_SIZE,
@@ -437,6 +444,72 @@ def workload_mixed8b(args) -> int:
     return 0
 
 
+def dafidra_config(width, heads, kv_heads, head_dim, ff, vocab, layers, window=1024, experts=16, top=4):
+    """A Dafidra of Llama-like layer sizes: attention as the Llama's, a matrix memory of heads / 4 heads with keys of
+    head_dim and values of 2 * head_dim, feed-forwards alternately dense (ff) and routed (``experts`` of ff / top,
+    ``top`` per token, in four groups of which two are kept)."""
+    left = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5, mask={"size": window},
+                q_temp={"coef": 0.5, "every": 128})
+    right = dict(heads=max(1, heads // 4), dim=head_dim, vdim=2 * head_dim, gate_cap=12.0)
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    return {"architecture": "Dafidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "layers": [{"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": dense if i % 2 == 0 else moe}
+                       for i in range(layers)]}
+
+
+def workload_dafidra(args) -> int:
+    """Dafidra beside a Llama of equal width, depth and vocabulary (see the module text)."""
+    import gc
+
+    import torch
+
+    layers = args.layers or 4
+    context = args.context
+    sizes = {"1b": MODEL, "3b": MODEL_3B}
+    results = {}
+    if args.only:       # for profiles: the Dafidra of the first size alone, a prompt or decode steps
+        b = sizes["1b"]
+        daf = dafidra_config(b["hidden_size"], b["num_attention_heads"], b["num_key_value_heads"], b["head_dim"],
+                             b["intermediate_size"], b["vocab_size"], layers)
+        runner, _cfg = make_runner(daf, layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                   max_model_len=max(context, PREFILL_TOKENS) + 64)
+        if args.only == "prefill":
+            sec = time_prefill(runner, PREFILL_TOKENS, max(1, args.steps // 8))
+            print(json.dumps({"only": "prefill", "model": "dafidra_1b", "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3)}), flush=True)
+        else:
+            sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context)
+            print(json.dumps({"only": "decode", "model": "dafidra_1b", "batch": args.batch, "ms_per_step": round(sec * 1e3, 4)}), flush=True)
+        return 0
+    for name, base in sizes.items():
+        daf = dafidra_config(base["hidden_size"], base["num_attention_heads"], base["num_key_value_heads"], base["head_dim"],
+                             base["intermediate_size"], base["vocab_size"], layers)
+        for what, raw in (("dafidra", daf), ("llama", dict(base, tie_word_embeddings=False))):
+            runner, _cfg = make_runner(raw, layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                       max_model_len=max(context, PREFILL_TOKENS) + 64)
+            psec = time_prefill(runner, PREFILL_TOKENS, 3)
+            dsec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context)
+            results[f"{what}_{name}"] = {"prefill_ms": round(psec * 1e3, 3), "prefill_tok_per_s": round(PREFILL_TOKENS / psec, 1),
+                                         "decode_ms_per_step": round(dsec * 1e3, 4), "decode_tok_per_s": round(args.batch / dsec, 1),
+                                         "graphs": len(runner._graphs)}
+            del runner
+            gc.collect()
+            torch.cuda.empty_cache()
+    first = results["dafidra_1b"]
+    line = {
+        "metric": f"decode tok/s at batch {args.batch}, context {context} (Dafidra at Llama 3.2 1B layer sizes, {layers} layers, random weights)",
+        "value": first["decode_tok_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "dafidra-at-llama-sizes", "layers": layers, "global_batch": args.batch, "seq_len": context,
+                   "prefill_tokens": PREFILL_TOKENS, "window": 1024, "experts": 16, "top": 4, "kv_block": BLOCK_SIZE,
+                   "parallelism": "single-gpu"},
+        "models": results,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -445,7 +518,7 @@ def main() -> int:
     ap.add_argument("--batch", default="8,1,64",
                     help="batch sizes of the decode steps: the first is the headline's, the others become points")
     ap.add_argument("--context", type=int, default=CONTEXT, help="context length that the decode steps end at")
-    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b"], default="decode1b")
+    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra"], default="decode1b")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -477,6 +550,8 @@ def main() -> int:
         return workload_serve3b(args)
     if args.workload == "mixed8b":
         return workload_mixed8b(args)
+    if args.workload == "dafidra":
+        return workload_dafidra(args)
     args.layers = args.layers or MODEL["num_hidden_layers"]
     elem = 2 if args.dtype == "bf16" else 4
     big = args.batch if (args.no_points or args.only) else max(batches)

@@ -170,13 +170,13 @@ __device__ inline void store_new_kv(const DecodeSource& src, long row, int g, in
   }
 }
 
-template <int HD, bool FUSED>
+template <int HD, bool FUSED, bool OPT = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_decode_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride, DecodeSource src,
     const bf16_t* k_cache, const bf16_t* v_cache,   // not restrict: the fused kernel stores into them
     const int* __restrict__ block_table,
     int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of, const int* __restrict__ req_ids,
-    int nh, int nkv, int page_size, float scale, int window, long num_pages, float* __restrict__ part) {
+    int nh, int nkv, int page_size, float scale, int window, long num_pages, float* __restrict__ part, AttnOptions opt) {
   const int lane = threadIdx.x, lr = lane % 16, lg = lane / 16;
   const int split = blockIdx.x, splits = gridDim.x, g = blockIdx.y;
   // the z-th request of this launch: all of the step's requests, or the listed ones (a step
@@ -194,6 +194,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   const bool valid = lr < G;     // the other columns are padding: computed on zeros, never stored
   st.pos[0] = p;
   st.lo[0] = lo;
+  st.bias[0] = (OPT && valid && opt.slopes) ? opt.slopes[g * G + lr] / scale : 0.f;
   // this wave's keys: chunk `split` of the 32-key chunks between lo and p
   const int first_chunk = lo / 32, last_chunk = p / 32;
   const int chunks = last_chunk - first_chunk + 1;
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
       __threadfence_block();
     }
   }
-  attn_walk<HD, 1>(st, c0, c1, (lo + 31) / 32, (p + 1) / 32 - 1, k_cache, v_cache, bt, table_width, kv_len, nkv, g,
+  attn_walk<HD, 1, OPT>(st, c0, c1, (lo + 31) / 32, (p + 1) / 32 - 1, k_cache, v_cache, bt, table_width, kv_len, nkv, g,
                    page_size, num_pages, scale * PI_LOG2E, lane, [&]() {
                      // while the first keys and values are on their way
                      if constexpr (!FUSED) {
@@ -225,7 +226,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   const int head = g * G + lr;
   if (splits == 1) {
     if (valid) {
-      const float inv = 1.0f / st.l[0];
+      float inv = 1.0f / st.l[0];
+      if (OPT) {
+        if (opt.sinks) inv = sink_inverse(st.l[0], st.m[0] * (scale * PI_LOG2E), opt.sinks[head]);
+        if (opt.gate) inv *= opt.gate[row * nh + head];
+      }
 #pragma unroll
       for (int db = 0; db < HD / 16; ++db) {
         uint2 w;
@@ -253,16 +258,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
 
 // Merge the key ranges of one (request, head) by one wave: lane d owns features d, d + 64, ..
 // Ranges are added in range order; an empty range (m = -inf) counts nothing.
+// sink2: the head's sink in base-2 units, joining the sum of weights once (-inf: none); gate: a
+// factor for the finished output.
 template <int HD>
-__device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base, int splits, int lane) {
+__device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base, int splits, int lane, float sink2 = -INFINITY,
+                                      float gate = 1.0f) {
   const int rec = HD + 4;
   constexpr int NF = (HD + 63) / 64;     // features per lane
   // lane s holds range s (splits <= 64): maxima, weights and the total in parallel
   const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
   const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
-  const float m_tot = wave_max(ms);
+  const float m_tot = fmaxf(wave_max(ms), sink2);
   const float w = range_weight(ms, m_tot);
-  float l_tot = 0.f;
+  float l_tot = range_weight(sink2, m_tot);
   float acc[NF];
 #pragma unroll
   for (int i = 0; i < NF; ++i) acc[i] = 0.f;
@@ -286,7 +294,7 @@ __device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base,
   }
 #pragma unroll
   for (int i = 0; i < NF; ++i)
-    if (lane + i * 64 < HD) o[lane + i * 64] = from_float<bf16_t>(range_finish(acc[i], l_tot));
+    if (lane + i * 64 < HD) o[lane + i * 64] = from_float<bf16_t>(range_finish(acc[i], l_tot) * gate);
 }
 
 // One wave per (request, head).
@@ -295,22 +303,23 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
                                                                const int* __restrict__ q_start,
                                                                const int* __restrict__ req_ids,
                                                                const int* __restrict__ rows,
-                                                               const float* __restrict__ part, int nh, int splits) {
+                                                               const float* __restrict__ part, int nh, int splits, AttnOptions opt) {
   const int head = blockIdx.x;
   // where the result goes: the token row of request r (decode), or a listed row (cut tiles)
   const int r = req_ids ? req_ids[blockIdx.y] : (int)blockIdx.y;
   const long out_row = rows ? rows[blockIdx.y] : q_start[r];
   combine_ranges<HD>(out + out_row * out_stride + (long)head * HD, part + ((long)blockIdx.y * nh + head) * splits * (HD + 4),
-                     splits, threadIdx.x);
+                     splits, threadIdx.x, opt.sinks ? opt.sinks[head] * PI_LOG2E : -INFINITY,
+                     opt.gate ? opt.gate[out_row * nh + head] : 1.0f);
 }
 
 // One wave per (row of `part`, head): rows are a launch's requests (results to the requests'
 // token rows) or listed token rows.
 static int launch_combine(void* out, long out_stride, const int* q_start, const int* req_ids, const int* rows, int Z,
-                          const void* part, int nh, int hd, int splits, hipStream_t stream) {
+                          const void* part, int nh, int hd, int splits, hipStream_t stream, AttnOptions opt = AttnOptions{nullptr, nullptr, nullptr}) {
   const dim3 grid(nh, Z), block(64);
 #define GO(H) hipLaunchKernelGGL(attention_combine_kernel<H>, grid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, rows, \
-                                 (const float*)part, nh, splits)
+                                 (const float*)part, nh, splits, opt)
   switch (hd) {
     case 16: GO(16); break;
     case 32: GO(32); break;
@@ -341,7 +350,9 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
                          const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                          const int* q_start, const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd,
                          int page_size, float scale, int window, long num_pages, int splits, void* part, long part_elems,
-                         bool merge, hipStream_t stream) {
+                         bool merge, hipStream_t stream, AttnOptions opt = AttnOptions{nullptr, nullptr, nullptr}) {
+  const bool with_options = opt.slopes || opt.sinks || opt.gate;
+  PI_REQUIRE(!with_options || (!fused && merge && scale > 0.f), "attention_decode: heads with options take the separate kernels, merged here, and a positive scale");
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
   PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_decode: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(!fused || hd == 64 || hd == 128, "attention_decode: the kernel that starts from the projection takes head_dim 64 or 128, not %d", hd);
@@ -355,9 +366,31 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
   const dim3 grid(splits, nkv, R), block(64);
 #define GO(H, F) hipLaunchKernelGGL((attention_decode_kernel<H, F>), grid, block, 0, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                     q_stride, src, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
-                                    kv_len, req_ids, nh, nkv, page_size, scale, window, num_pages, (float*)part)
+                                    kv_len, req_ids, nh, nkv, page_size, scale, window, num_pages, (float*)part, opt)
+#define GO_OPT(H) hipLaunchKernelGGL((attention_decode_kernel<H, false, true>), grid, block, 0, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
+                                    q_stride, src, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
+                                    kv_len, req_ids, nh, nkv, page_size, scale, window, num_pages, (float*)part, opt)
   if (fused) { if (hd == 64) GO(64, true); else GO(128, true); }
-  else {
+  else if (with_options) {
+    switch (hd) {
+      case 16: GO_OPT(16); break;
+      case 32: GO_OPT(32); break;
+      case 48: GO_OPT(48); break;
+      case 64: GO_OPT(64); break;
+      case 80: GO_OPT(80); break;
+      case 96: GO_OPT(96); break;
+      case 112: GO_OPT(112); break;
+      case 128: GO_OPT(128); break;
+      case 144: GO_OPT(144); break;
+      case 160: GO_OPT(160); break;
+      case 176: GO_OPT(176); break;
+      case 192: GO_OPT(192); break;
+      case 208: GO_OPT(208); break;
+      case 224: GO_OPT(224); break;
+      case 240: GO_OPT(240); break;
+      default: GO_OPT(256); break;
+    }
+  } else {
     switch (hd) {
       case 16: GO(16, false); break;
       case 32: GO(32, false); break;
@@ -378,9 +411,10 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
     }
   }
 #undef GO
+#undef GO_OPT
   if (pi_check_launch("attention_decode")) return -1;
   // merge == false: the caller's next kernel merges the ranges itself (nothing is in `out` then)
-  if (splits > 1 && merge) return launch_combine(out, out_stride, q_start, req_ids, nullptr, R, part, nh, hd, splits, stream);
+  if (splits > 1 && merge) return launch_combine(out, out_stride, q_start, req_ids, nullptr, R, part, nh, hd, splits, stream, opt);
   return 0;
 }
 
@@ -388,9 +422,10 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
                                    const void* v_cache, const int* block_table, int table_width, const int* q_start,
                                    const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd, int page_size,
                                    float scale, int window, long num_pages, int splits, void* part, long part_elems,
-                                   hipStream_t stream) {
+                                   const float* slopes, const float* sinks, const float* gate, hipStream_t stream) {
   return launch_decode(false, DecodeSource{}, out, out_stride, q, q_stride, k_cache, v_cache, block_table, table_width, q_start,
-                       kv_len, req_ids, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, true, stream);
+                       kv_len, req_ids, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, true, stream,
+                       AttnOptions{slopes, sinks, gate});
 }
 
 // The same for a step of single tokens only (T == R tokens, request r at row q_start[r]),
@@ -439,7 +474,7 @@ extern "C" int pi_attention_decode_fused(void* out, long out_stride, const void*
 // Merge partial results that the tile kernel wrote for `Z` tokens whose tiles' keys were cut in
 // `cuts` shares: part [Z, nh, cuts, hd + 4]; token z's result goes to row rows[z] of out.
 extern "C" int pi_attention_combine_rows(void* out, long out_stride, const int* rows, int Z, const void* part, int nh, int hd,
-                                         int cuts, hipStream_t stream) {
+                                         int cuts, const float* sinks, const float* gate, hipStream_t stream) {
   PI_REQUIRE(Z > 0 && Z <= 65535 && nh > 0 && cuts >= 2 && cuts <= 64 && rows && part, "attention_combine_rows: bad arguments (%d tokens, %d heads, %d cuts)", Z, nh, cuts);
-  return launch_combine(out, out_stride, nullptr, nullptr, rows, Z, part, nh, hd, cuts, stream);
+  return launch_combine(out, out_stride, nullptr, nullptr, rows, Z, part, nh, hd, cuts, stream, AttnOptions{nullptr, sinks, gate});
 }

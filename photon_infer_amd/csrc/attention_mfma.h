@@ -44,7 +44,28 @@ struct AttnState {
   float l[CB];          // the same as a scalar, set by attn_finish
   int pos[CB];          // last visible key of the column
   int lo[CB];           // first visible key of the column
+  float bias[CB];       // distance bias of the column's head per key of distance, in raw score units
+                        // (slope / scale); read only by the BIAS variants of the arithmetic
 };
+
+// Options of a head beyond plain softmax attention, each off when its pointer is null:
+//   slopes [heads]: slope * (p - t) is taken off the scaled score of key t for the query at p;
+//   sinks  [heads]: exp(sink) joins the softmax's denominator once (no key, no value, no scale, no bias);
+//   gate   [tokens, heads] float32: multiplies the head's output.
+struct AttnOptions {
+  const float* slopes;
+  const float* sinks;
+  const float* gate;
+};
+
+// The sink joins a column's sum of weights l, which is relative to the base-2 reference m2
+// (-inf: nothing seen): returns the factor for the un-normalised output, 1 / (l' ) included.
+__device__ inline float sink_inverse(float l, float m2, float sink) {
+  const float s2 = sink * PI_LOG2E;
+  const float mt = fmaxf(m2, s2);
+  const float a = (m2 == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m2 - mt);
+  return a / (l * a + __builtin_amdgcn_exp2f(s2 - mt));
+}
 
 template <int HD>
 struct KVChunk {
@@ -191,7 +212,7 @@ __device__ inline void attn_load(KVChunk<HD>& kv, const ChunkPages& cp, const bf
 // st.m is a column's reference score (raw, before the softmax scale): at least the largest
 // score seen minus the slack.  Moving it costs a pass over the accumulators, so it only moves
 // when some column of the wave needs it.
-template <int HD, int CB, bool MASKED, class KV>
+template <int HD, int CB, bool MASKED, class KV, bool BIAS = false>
 __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0, float scale_log2, int lane) {
   const int lg = lane / 16;
   f32x4_t s[2][CB];
@@ -202,6 +223,11 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
       f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < HeadFrags<HD>::KS; ++ks) acc = mfma16(kv.key(t, ks), st.q[c][ks], acc);
+      if (BIAS) {   // the distance bias joins the raw score before anything looks at it
+        const float base = st.bias[c] * (float)(k0 + t * 16 + lg * 4 - st.pos[c]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += __builtin_fmaf(st.bias[c], (float)i, base);
+      }
       s[t][c] = acc;
     }
   const float slack = PI_RESCALE_SLACK / scale_log2;
@@ -275,8 +301,9 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
 // formed first, then one test decides whether any column's reference has to move, then the
 // weights and the accumulation run as straight-line code: matrix and vector instructions of
 // different chunks and columns can overlap, and the test costs one branch per group.
-template <int HD, int CB, int NJ>
-__device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* from, int chunk_stride, float scale_log2) {
+template <int HD, int CB, int NJ, bool BIAS = false>
+__device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* from, int chunk_stride, float scale_log2,
+                                          int key0 = 0, int lane = 0) {
   // The key fragments of a chunk are read from LDS while the products of the chunk before it
   // run; the scheduler is told so, or it reads each fragment right before its use to save
   // registers and the wave waits for LDS sixteen times per group.
@@ -303,6 +330,18 @@ __device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* 
     }
     if (j + 1 < NJ) __builtin_amdgcn_sched_group_barrier(0x100, KF, 0);   // LDS reads of the next chunk
     __builtin_amdgcn_sched_group_barrier(0x008, KF * CB, 0);               // this chunk's products
+  }
+  if (BIAS) {
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      const float base = st.bias[c] * (float)(key0 + (lane / 16) * 4 - st.pos[c]);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[j][t][c][i] += __builtin_fmaf(st.bias[c], (float)(j * 32 + t * 16 + i), base);
+    }
   }
   const float slack = PI_RESCALE_SLACK / scale_log2;
   float mx[CB];
@@ -365,10 +404,10 @@ __device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* 
   }
 }
 
-template <int HD, int CB, class KV>
+template <int HD, int CB, class KV, bool BIAS = false>
 __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0, float scale_log2, bool masked, int lane) {
-  if (masked) attn_compute<HD, CB, true, KV>(st, kv, k0, scale_log2, lane);
-  else attn_compute<HD, CB, false, KV>(st, kv, k0, scale_log2, lane);
+  if (masked) attn_compute<HD, CB, true, KV, BIAS>(st, kv, k0, scale_log2, lane);
+  else attn_compute<HD, CB, false, KV, BIAS>(st, kv, k0, scale_log2, lane);
 }
 
 // Walk chunks c0 .. c1-1 (32 keys each) with the next chunk's loads in flight during the
@@ -376,7 +415,7 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
 // are known to be fully visible to every column.
 // `meanwhile` is called once the first chunk's loads are on their way (also when the range is
 // empty): work that the walk needs but the loads do not, such as fetching the queries.
-template <int HD, int CB, class Meanwhile>
+template <int HD, int CB, bool BIAS = false, class Meanwhile>
 __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int first_unmasked, int last_unmasked,
                                  const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                                  const int* __restrict__ bt, int table_width, int kv_len, int nkv, int g, int page_size,
@@ -408,10 +447,10 @@ __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int firs
   for (int c = c0; c < c1; c += 2) {
     pa = cur.next();
     attn_load<HD>(b, pb, k_cache, v_cache, off, nkv, g, page_size, num_pages);
-    attn_compute<HD, CB>(st, a, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
+    attn_compute<HD, CB, KVChunk<HD>, BIAS>(st, a, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
     pb = cur.next();
     attn_load<HD>(a, pa, k_cache, v_cache, off, nkv, g, page_size, num_pages);
-    if (c + 1 < c1) attn_compute<HD, CB>(st, b, (c + 1) * 32, scale_log2, c + 1 < first_unmasked || c + 1 > last_unmasked, lane);
+    if (c + 1 < c1) attn_compute<HD, CB, KVChunk<HD>, BIAS>(st, b, (c + 1) * 32, scale_log2, c + 1 < first_unmasked || c + 1 > last_unmasked, lane);
   }
 }
 

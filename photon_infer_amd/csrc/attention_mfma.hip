@@ -21,14 +21,15 @@
 #endif
 
 // NCH: chunks of 32 keys per round (4, or 2 for the large heads)
-template <int HD, int CB, int NCH>
+// OPT: the heads have options (AttnOptions: distance bias, sink, output gate).
+template <int HD, int CB, int NCH, bool OPT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_tiles_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of,
     const int* __restrict__ tile_req, const int* __restrict__ tile_q0, const int* __restrict__ tile_cut,
     const int* __restrict__ tile_z0, float* __restrict__ part, const int* __restrict__ order, int rounds, int nh,
-    int nkv, int page_size, float scale, int window, long num_pages_l, int TQ) {
+    int nkv, int page_size, float scale, int window, long num_pages_l, int TQ, AttnOptions opt) {
   constexpr int KS = HeadFrags<HD>::KS;
   constexpr int F = 2 * KS + HD / 16;             // 16-byte operand fragments per lane and 32 keys: keys, then values
   constexpr int KEYS_PER_ROUND = NCH * 32;
@@ -90,6 +91,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
       // padding columns are computed on zeros, see everything and are never stored
       st.pos[c] = valid[c] ? pos0 + tok : 0x7fffffff;
       st.lo[c] = valid[c] ? first_key(pos0 + tok) : 0;
+      st.bias[c] = (OPT && valid[c] && opt.slopes) ? opt.slopes[heads[c]] / scale : 0.f;
       attn_load_q(st, c, q, q_stride, rows[c], heads[c], valid[c], lane);
     }
 
@@ -136,8 +138,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
       const bool missing = __builtin_amdgcn_ballot_w64(lane < 2 * NCH && !(&present[buf][0][0])[lane % 8]) != 0;
       constexpr int NJ = NCH < PLAIN_NJ ? NCH : PLAIN_NJ;
       if (active && !missing && round0 >= see_all_lo && round0 + KEYS_PER_ROUND - 1 <= see_all_hi) {
-        attn_compute_plain<HD, CB, NJ>(st, staged + (buf * NCH * F) * 64 + lane, F * 64, scale_log2);
-        if (NJ < NCH) attn_compute_plain<HD, CB, NJ>(st, staged + ((buf * NCH + 2) * F) * 64 + lane, F * 64, scale_log2);
+        attn_compute_plain<HD, CB, NJ, OPT>(st, staged + (buf * NCH * F) * 64 + lane, F * 64, scale_log2, round0, lane);
+        if (NJ < NCH) attn_compute_plain<HD, CB, NJ, OPT>(st, staged + ((buf * NCH + 2) * F) * 64 + lane, F * 64, scale_log2, round0 + 64, lane);
       } else if (active) {
 #pragma unroll 1
         for (int j = 0; j < NCH; ++j) {
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
           kv.have[0] = __builtin_amdgcn_readfirstlane(present[buf][j][0]) != 0;
           kv.have[1] = __builtin_amdgcn_readfirstlane(present[buf][j][1]) != 0;
           const bool masked = key0 < see_all_lo || key0 + 31 > see_all_hi || !kv.have[0] || !kv.have[1];
-          attn_compute<HD, CB, StagedChunk<HD>>(st, kv, key0, scale_log2, masked, lane);
+          attn_compute<HD, CB, StagedChunk<HD>, OPT>(st, kv, key0, scale_log2, masked, lane);
         }
       }
       stash(buf ^ 1);
@@ -177,7 +179,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
 #pragma unroll
     for (int c = 0; c < CB; ++c) {
       if (!valid[c]) continue;
-      const float inv = 1.0f / st.l[c];
+      float inv = 1.0f / st.l[c];
+      if (OPT) {
+        if (opt.sinks) inv = sink_inverse(st.l[c], st.m[c] * scale_log2, opt.sinks[heads[c]]);
+        if (opt.gate) inv *= opt.gate[rows[c] * nh + heads[c]];
+      }
       bf16_t* o = out + rows[c] * out_stride + (long)heads[c] * HD + lg * 4;
 #pragma unroll
       for (int db = 0; db < HD / 16; ++db) {
@@ -209,7 +215,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
                                          const int* kv_len, const int* tile_req, const int* tile_q0, const int* tile_cut,
                                          const int* tile_z0, void* part, const int* order, int rounds, int seats, int nh,
                                          int nkv, int hd, int page_size, float scale, int window, long num_pages,
-                                         hipStream_t stream) {
+                                         const float* slopes, const float* sinks, const float* gate, hipStream_t stream) {
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
   PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_prefill: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
@@ -220,18 +226,26 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
   const dim3 grid(nkv, seats), block(256);
-#define GO(H, C, N)                                                                                                                          \
+  const AttnOptions opt{slopes, sinks, gate};
+  const bool with_options = slopes || sinks || gate;
+  PI_REQUIRE(!with_options || scale > 0.f, "attention_prefill: a distance bias needs a positive scale");
+#define GO(H, C, N)                    \
+  do {                                 \
+    if (with_options) GO1(H, C, N, true); \
+    else GO1(H, C, N, false);          \
+  } while (0)
+#define GO1(H, C, N, O)                                                                                                                          \
   do {                                                                                                                                     \
     static bool configured = false;                                                                                                        \
     if (!configured) {                                                                                                                     \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_tiles_kernel<H, C, N>),                                      \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_tiles_kernel<H, C, N, O>),                                    \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                            \
       if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));            \
       configured = true;                                                                                                                   \
     }                                                                                                                                      \
-    hipLaunchKernelGGL((attention_tiles_kernel<H, C, N>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride,     \
+    hipLaunchKernelGGL((attention_tiles_kernel<H, C, N, O>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride,     \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, kv_len, tile_req, tile_q0,       \
-                       tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, window, num_pages, TQ);                  \
+                       tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, window, num_pages, TQ, opt);             \
   } while (0)
   switch (hd) {
     case 16: GO(16, 2, 4); break;
@@ -252,5 +266,6 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
     default: GO(256, 1, 2); break;
   }
 #undef GO
+#undef GO1
   return pi_check_launch("attention_prefill_mfma");
 }

@@ -143,7 +143,9 @@ __device__ inline __amdgpu_buffer_rsrc_t operand_descriptor(const bf16_t* operan
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
                                                         const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
-                                                        int tiles_n, int k_per_split) {
+                                                        int tiles_n, int k_per_split, const int* __restrict__ group_of_tile,
+                                                        const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
+                                                        long group_stride) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   constexpr int ROW = BK;                   // rows of 128 bytes, no padding (see the large-tile kernel)
   constexpr int TILE = BM * ROW;
@@ -168,6 +170,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   } else {
     tile_m = blockIdx.x / tiles_n;
     tile_n = blockIdx.x % tiles_n;
+  }
+  // Grouped: the rows are sorted by group (a routed feed-forward's experts) and cut into tiles of
+  // up to 128 rows of one group; tile t multiplies rows tile_row0[t] .. + tile_rows[t] - 1 with the
+  // matrix of group group_of_tile[t] (W + group * group_stride).  The list lives on the device
+  // and is as long as the worst case; unused entries (-1) end their blocks at once.
+  if (group_of_tile) {
+    const int t = blockIdx.x / tiles_n;
+    const int grp = group_of_tile[t];
+    if (grp < 0) return;
+    const long r0 = tile_row0[t];
+    tile_m = 0;
+    tile_n = blockIdx.x % tiles_n;
+    M = tile_rows[t];
+    A += r0 * lda;
+    W += (long)grp * group_stride;
+    Cv = reinterpret_cast<char*>(Cv) + r0 * ldc * (EPI == EPI_BF16 || EPI == EPI_SWIGLU ? 2 : 4);
   }
   const long m0 = (long)tile_m * BM, n0 = (long)tile_n * BN;
 
@@ -490,8 +508,53 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
   }
   const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
   hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles_m * tiles_n, splits), dim3(256), kLdsBytes, stream, C, ldc,
-                     (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, tiles_n, kps);
+                     (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, tiles_n, kps, (const int*)nullptr, (const int*)nullptr,
+                     (const int*)nullptr, 0L);
   return pi_check_launch("gemm_mfma");
+}
+
+// Rows of a grouped product's tiles (the 128 x 128 kernel's block tile).
+extern "C" int pi_gemm_mfma_group_tile_rows() { return BM; }
+
+// C[row, :] = A[row, :] . W[group of row]^T over a device-side list of `tiles` row tiles (see the
+// kernel); W is [groups, N, K] with `group_stride` elements from one group's matrix to the next.
+// epilogue: 0 store bf16, 1 store f32, 3 SwiGLU (every group's rows interleaved by 16; C is [rows, N / 2] bf16).
+template <int EPI>
+static int launch_grouped(void* C, long ldc, const void* A, long lda, const void* W, long ldw, long group_stride,
+                          const int* group_of_tile, const int* tile_row0, const int* tile_rows, int tiles, int N, int K,
+                          hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_kernel<EPI>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    if (e != hipSuccess) return pi_fail("gemm_mfma: cannot reserve %zu bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
+    configured = true;
+  }
+  const int tiles_n = ceil_div(N, BN);
+  hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles * tiles_n, 1), dim3(256), kLdsBytes, stream, C, ldc,
+                     (const bf16_t*)A, lda, (const bf16_t*)W, ldw, BM, N, K, tiles_n, K, group_of_tile, tile_row0, tile_rows,
+                     group_stride);
+  return pi_check_launch("gemm_mfma_grouped");
+}
+
+extern "C" int pi_gemm_mfma_grouped(void* C, int epilogue, long ldc, const void* A, long lda, const void* W, long ldw,
+                                    long group_stride, const int* group_of_tile, const int* tile_row0, const int* tile_rows,
+                                    int tiles, int N, int K, hipStream_t stream) {
+  PI_REQUIRE(tiles >= 0 && N > 0 && K > 0, "gemm_mfma_grouped: bad sizes tiles=%d N=%d K=%d", tiles, N, K);
+  PI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && group_stride % 8 == 0, "gemm_mfma_grouped: K (%d) and strides must be multiples of 8", K);
+  PI_REQUIRE(256 * lda < (1L << 29) && 256 * ldw < (1L << 29), "gemm_mfma_grouped: row strides (%ld, %ld) are too long", lda, ldw);
+  PI_REQUIRE(ldc > 0 && ldc < (1L << 23), "gemm_mfma_grouped: the result's row stride (%ld) is too long", ldc);
+  PI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mfma_grouped: operands must be 16-byte aligned");
+  PI_REQUIRE(epilogue != EPI_SWIGLU || N % 32 == 0, "gemm_mfma_grouped: the SwiGLU epilogue needs N (%d) to be a multiple of 32", N);
+  PI_REQUIRE((long)tiles * ceil_div(N, BN) < 2147483647L, "gemm_mfma_grouped: too many tiles");
+  PI_REQUIRE(group_of_tile && tile_row0 && tile_rows, "gemm_mfma_grouped: the tile list is missing");
+  if (tiles == 0) return 0;
+  switch (epilogue) {
+    case EPI_BF16: return launch_grouped<EPI_BF16>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, stream);
+    case EPI_F32: return launch_grouped<EPI_F32>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, stream);
+    case EPI_SWIGLU: return launch_grouped<EPI_SWIGLU>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, stream);
+  }
+  return pi_fail("gemm_mfma_grouped: unknown epilogue %d", epilogue);
 }
 
 // Pieces a k-split into `splits` makes (the kernel rounds a split's range up to whole slabs).

@@ -11,7 +11,7 @@
 #include "common.h"
 
 #define RE_MAX_EXPERTS 1024
-#define RE_TILE 64          // rows of a tile of the grouped products
+#define RE_TILE 64          // rows of a tile of the general grouped product (the most it takes)
 
 // (value, index) arg max over a wave; equal values: the lower index
 __device__ inline void wave_argmax(float& v, int& idx) {
@@ -117,12 +117,13 @@ extern "C" int pi_route(int* ids, float* weights, const float* logits, long logi
 // ---------------------------------------------------------------- entries grouped by expert
 // N entries (entry = token * top + choice) with their expert ids -> rows in expert order:
 //   row_entry[row] = entry, entry_row[entry] = row (entries of one expert keep their order),
-//   tiles of up to RE_TILE rows that never straddle two experts: tile_expert[i] (-1: unused),
-//   tile_row0[i], tile_rows[i]; max_tiles = ceil(N / RE_TILE) + E bounds their number.
+//   tiles of up to `tile` rows that never straddle two experts: tile_expert[i] (-1: unused),
+//   tile_row0[i], tile_rows[i]; max_tiles = ceil(N / tile) + E bounds their number.
 // One block of 1024 threads; wave w places the experts w, w + 16, ...
 __global__ __launch_bounds__(1024) void group_entries_kernel(const int* __restrict__ ids, int N, int E, int* __restrict__ row_entry,
                                                              int* __restrict__ entry_row, int* __restrict__ tile_expert,
-                                                             int* __restrict__ tile_row0, int* __restrict__ tile_rows, int max_tiles) {
+                                                             int* __restrict__ tile_row0, int* __restrict__ tile_rows, int max_tiles,
+                                                             int tile) {
   __shared__ int count[RE_MAX_EXPERTS];
   __shared__ int start[RE_MAX_EXPERTS + 1];
   __shared__ int tstart[RE_MAX_EXPERTS + 1];
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(1024) void group_entries_kernel(const int* __restri
       start[e] = acc;
       tstart[e] = tacc;
       acc += count[e];
-      tacc += (count[e] + RE_TILE - 1) / RE_TILE;
+      tacc += (count[e] + tile - 1) / tile;
     }
     start[E] = acc;
     tstart[E] = tacc;
@@ -152,11 +153,11 @@ __global__ __launch_bounds__(1024) void group_entries_kernel(const int* __restri
     tile_rows[i] = 0;
   }
   for (int e = wave; e < E; e += 16) {
-    for (int i = lane; i < (count[e] + RE_TILE - 1) / RE_TILE; i += PI_WAVE) {
+    for (int i = lane; i < (count[e] + tile - 1) / tile; i += PI_WAVE) {
       tile_expert[tstart[e] + i] = e;
-      tile_row0[tstart[e] + i] = start[e] + i * RE_TILE;
-      const int left = count[e] - i * RE_TILE;
-      tile_rows[tstart[e] + i] = left < RE_TILE ? left : RE_TILE;
+      tile_row0[tstart[e] + i] = start[e] + i * tile;
+      const int left = count[e] - i * tile;
+      tile_rows[tstart[e] + i] = left < tile ? left : tile;
     }
     int placed = start[e];
     for (int i0 = 0; i0 < N; i0 += PI_WAVE) {
@@ -174,12 +175,12 @@ __global__ __launch_bounds__(1024) void group_entries_kernel(const int* __restri
 }
 
 extern "C" int pi_group_entries(const int* ids, int N, int E, int* row_entry, int* entry_row, int* tile_expert, int* tile_row0,
-                                int* tile_rows, int max_tiles, hipStream_t stream) {
-  PI_REQUIRE(N >= 0 && E > 0 && E <= RE_MAX_EXPERTS, "grouping: bad sizes N=%d E=%d", N, E);
-  PI_REQUIRE(max_tiles >= (N + RE_TILE - 1) / RE_TILE + E, "grouping: room for %d tiles is too little", max_tiles);
+                                int* tile_rows, int max_tiles, int tile, hipStream_t stream) {
+  PI_REQUIRE(N >= 0 && E > 0 && E <= RE_MAX_EXPERTS && tile > 0, "grouping: bad sizes N=%d E=%d tile=%d", N, E, tile);
+  PI_REQUIRE(max_tiles >= (N + tile - 1) / tile + E, "grouping: room for %d tiles is too little", max_tiles);
   if (N == 0) return 0;
   hipLaunchKernelGGL(group_entries_kernel, dim3(1), dim3(1024), 0, stream, ids, N, E, row_entry, entry_row, tile_expert, tile_row0,
-                     tile_rows, max_tiles);
+                     tile_rows, max_tiles, tile);
   return pi_check_launch("group_entries");
 }
 
@@ -222,43 +223,47 @@ __global__ __launch_bounds__(256) void grouped_gemm_general_kernel(TC* __restric
   __shared__ float Ws[RG_K][RG_T + 4];
   const int tid = threadIdx.x;
   const int tx = tid % 16, ty = tid / 16;
-  const long m0 = tile_row0[blockIdx.y], n0 = (long)blockIdx.x * RG_T;
-  const int M = tile_rows[blockIdx.y];
+  const long n0 = (long)blockIdx.x * RG_T;
   const TW* We = W + (long)e * w_expert_stride;
-  float acc[4][4] = {};
-  for (int k0 = 0; k0 < K; k0 += RG_K) {
+  // a tile of more than RG_T rows (lists made for the matrix-core kernel) is walked in pieces
+  for (int sub = 0; sub < tile_rows[blockIdx.y]; sub += RG_T) {
+    const long m0 = tile_row0[blockIdx.y] + sub;
+    const int M = min(RG_T, tile_rows[blockIdx.y] - sub);
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += RG_K) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int idx = tid + i * 256;
+        const int row = idx / RG_K, kk = idx % RG_K;
+        const long n = n0 + row;
+        const int k = k0 + kk;
+        As[kk][row] = (row < M && k < K) ? to_float(A[(m0 + row) * lda + k]) : 0.f;
+        Ws[kk][row] = (n < N && k < K) ? to_float(We[n * ldw + k]) : 0.f;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < RG_K; ++kk) {
+        float a[4], w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+      }
+      __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int idx = tid + i * 256;
-      const int row = idx / RG_K, kk = idx % RG_K;
-      const long n = n0 + row;
-      const int k = k0 + kk;
-      As[kk][row] = (row < M && k < K) ? to_float(A[(m0 + row) * lda + k]) : 0.f;
-      Ws[kk][row] = (n < N && k < K) ? to_float(We[n * ldw + k]) : 0.f;
-    }
-    __syncthreads();
+      const int r = ty * 4 + i;
+      if (r >= M) continue;
 #pragma unroll
-    for (int kk = 0; kk < RG_K; ++kk) {
-      float a[4], w[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
-    }
-    __syncthreads();
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = ty * 4 + i;
-    if (r >= M) continue;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const long n = n0 + tx * 4 + j;
-      if (n < N) C[(m0 + r) * ldc + n] = from_float<TC>(acc[i][j]);
+      for (int j = 0; j < 4; ++j) {
+        const long n = n0 + tx * 4 + j;
+        if (n < N) C[(m0 + r) * ldc + n] = from_float<TC>(acc[i][j]);
+      }
     }
   }
 }

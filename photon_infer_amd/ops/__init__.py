@@ -427,10 +427,11 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise KernelError("attention: block table must be contiguous int32 [requests, width]")
     if T == 0:
         return
-    if _FAST and q.dtype == torch.bfloat16 and plain:
+    if _FAST and q.dtype == torch.bfloat16 and vd == head_dim and head_dim % 16 == 0 and (plain or scale > 0):
+        # the matrix-core kernels take heads whose values are as wide as their keys, options included
         from . import fast
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                                page_size, scale, window, pages, ws):
+                                page_size, scale, window, pages, ws, slopes, sinks, gate):
             return
     # a step of few tokens over long contexts: its keys cut into ranges, merged by a second kernel
     # (as many as the context-length bucket asks for, so that a step gives the same bits eagerly and replayed)
@@ -633,30 +634,39 @@ def route(logits: torch.Tensor, top: int, groups: int = 1, keep: int = 1, renorm
 
 
 class ExpertRows:
-    """A step's (token, choice) entries in expert order, and the tiles of the grouped products."""
+    """A step's (token, choice) entries in expert order, and the tiles of the grouped products
+    (``tile`` rows at most, none straddling two experts)."""
 
-    def __init__(self, row_entry, entry_row, tile_expert, tile_row0, tile_rows, top):
+    def __init__(self, row_entry, entry_row, tile_expert, tile_row0, tile_rows, top, tile):
         self.row_entry, self.entry_row = row_entry, entry_row
-        self.tile_expert, self.tile_row0, self.tile_rows, self.top = tile_expert, tile_row0, tile_rows, top
+        self.tile_expert, self.tile_row0, self.tile_rows, self.top, self.tile = tile_expert, tile_row0, tile_rows, top, tile
 
     @property
     def rows(self) -> int:
         return self.row_entry.numel()
 
 
-def group_entries(ids: torch.Tensor, num_experts: int) -> ExpertRows:
+def grouped_tile_rows(dtype: torch.dtype) -> int:
+    """Rows per tile of the grouped products that serve ``dtype``: the matrix-core kernel's block
+    tile for bfloat16, the general kernel's otherwise."""
+    if _FAST and dtype == torch.bfloat16 and _lib.build.MODULES["bf16"]:
+        return int(_lib.load("bf16").pi_gemm_mfma_group_tile_rows())
+    return int(_lib.load("core").pi_group_tile_rows())
+
+
+def group_entries(ids: torch.Tensor, num_experts: int, tile: Optional[int] = None) -> ExpertRows:
     """Sort the entries of ``ids`` (int32 [T, top]) by expert, on the device."""
     _gpu(ids)
     _i32(ids, "expert ids")
     N = ids.numel()
-    tile = int(_lib.load("core").pi_group_tile_rows())
+    tile = int(tile or _lib.load("core").pi_group_tile_rows())
     max_tiles = -(-N // tile) + num_experts
     meta = torch.empty(2 * N + 3 * max_tiles, dtype=torch.int32, device=ids.device)
     row_entry, entry_row = meta[:N], meta[N:2 * N]
     te, t0, tr = (meta[2 * N + i * max_tiles: 2 * N + (i + 1) * max_tiles] for i in range(3))
     _lib.call("core", "pi_group_entries", ids.data_ptr(), N, int(num_experts), row_entry.data_ptr(), entry_row.data_ptr(),
-              te.data_ptr(), t0.data_ptr(), tr.data_ptr(), max_tiles, _stream())
-    return ExpertRows(row_entry, entry_row, te, t0, tr, ids.shape[1])
+              te.data_ptr(), t0.data_ptr(), tr.data_ptr(), max_tiles, tile, _stream())
+    return ExpertRows(row_entry, entry_row, te, t0, tr, ids.shape[1], tile)
 
 
 def gather_rows(src: torch.Tensor, rows: ExpertRows) -> torch.Tensor:
@@ -670,6 +680,21 @@ def gather_rows(src: torch.Tensor, rows: ExpertRows) -> torch.Tensor:
     return out
 
 
+def _grouped_fast(out, a, w, rows: ExpertRows, epilogue: int) -> bool:
+    """The matrix-core grouped product, when the operands are what it takes."""
+    if not (_FAST and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _lib.build.MODULES["bf16"]):
+        return False
+    K = w.shape[2]
+    if K % 8 or _rows(a, "a") % 8 or a.data_ptr() % 16 or w.data_ptr() % 16 or (w.shape[1] * K) % 8:
+        return False
+    if rows.tile != int(_lib.load("bf16").pi_gemm_mfma_group_tile_rows()):
+        return False
+    _lib.call("bf16", "pi_gemm_mfma_grouped", out.data_ptr(), epilogue, _rows(out, "out"), a.data_ptr(), _rows(a, "a"), w.data_ptr(),
+              K, w.shape[1] * K, rows.tile_expert.data_ptr(), rows.tile_row0.data_ptr(), rows.tile_rows.data_ptr(),
+              rows.tile_expert.numel(), w.shape[1], K, _stream())
+    return True
+
+
 def grouped_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, rows: ExpertRows) -> None:
     """out[row] = a[row] @ w[expert of row]^T for rows in expert order; ``w`` is [experts, N, K]."""
     _gpu(out, a, w)
@@ -677,9 +702,30 @@ def grouped_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, rows: Expe
         raise KernelError(f"grouped product: shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
     if a.dtype != w.dtype:
         raise KernelError(f"grouped product: activations {a.dtype} and weights {w.dtype} must have one type")
+    if rows.rows == 0:
+        return
+    if out.dtype in (torch.bfloat16, torch.float32) and _grouped_fast(out, a, w, rows, 0 if out.dtype == torch.bfloat16 else 1):
+        return
     _lib.call("core", "pi_grouped_gemm_general", out.data_ptr(), _dt(out), _rows(out, "out"), a.data_ptr(), _dt(a), _rows(a, "a"),
               w.data_ptr(), _dt(w), w.shape[2], w.shape[1] * w.shape[2], rows.tile_expert.data_ptr(), rows.tile_row0.data_ptr(),
               rows.tile_rows.data_ptr(), rows.tile_expert.numel(), w.shape[1], w.shape[2], _stream())
+
+
+def grouped_gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, rows: ExpertRows, block: int = 0) -> None:
+    """out[row] = silu(a[row] @ Wg^T) * (a[row] @ Wu^T) with the row's expert's matrices: ``w_gate_up``
+    [experts, 2F, K] holds every expert's gate and up rows in halves (``block`` 0) or interleaved in
+    blocks of ``block`` rows.  With bfloat16 operands and blocks of 16 product and activation are one kernel."""
+    _gpu(out, a, w_gate_up)
+    F2 = w_gate_up.shape[1]
+    if out.shape != (rows.rows, F2 // 2) or out.dtype != a.dtype:
+        raise KernelError(f"grouped swiglu: out {tuple(out.shape)} does not match {rows.rows} x {F2 // 2}")
+    if rows.rows == 0:
+        return
+    if block == 16 and F2 % 32 == 0 and out.is_contiguous() and _grouped_fast(out, a, w_gate_up, rows, 3):
+        return
+    gu = torch.empty((rows.rows, F2), dtype=a.dtype, device=a.device)
+    grouped_gemm(gu, a, w_gate_up, rows)
+    swiglu(out, gu, block)
 
 
 def combine_choices(out: torch.Tensor, y: torch.Tensor, weights: torch.Tensor, rows: ExpertRows, accumulate: bool = False) -> None:

@@ -27,7 +27,7 @@ _SIGNATURES = {
         "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, P],
         "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, P],
         "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
-        "pi_group_entries": [P, I, I, P, P, P, P, P, I, P],
+        "pi_group_entries": [P, I, I, P, P, P, P, P, I, I, P],
         "pi_gather_rows": [P, P, I, P, I, I, I, P],
         "pi_grouped_gemm_general": [P, I, L, P, I, L, P, I, L, L, P, P, P, I, I, I, P],
         "pi_combine_choices": [P, P, P, P, I, I, I, I, P],
@@ -39,12 +39,13 @@ _SIGNATURES = {
     "bf16": {
         "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, I, P],
         "pi_gemm_mfma_pieces": [I, I],
+        "pi_gemm_mfma_grouped": [P, I, L, P, L, P, L, L, P, P, P, I, I, I, P],
         "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, I, P],
         "pi_splitk_reduce": [P, I, L, P, I, I, I, P],
         "pi_attention_tile_rows": [I, I, I],
-        "pi_attention_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, L, P],
-        "pi_attention_combine_rows": [P, L, P, I, P, I, I, I, P],
-        "pi_attention_decode": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
+        "pi_attention_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, L, P, P, P, P],
+        "pi_attention_combine_rows": [P, L, P, I, P, I, I, I, P, P, P],
+        "pi_attention_decode": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, L, I, P, L, P, P, P, P],
         "pi_attention_decode_fused": [P, L, P, L, P, I, I, I, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P],
         "pi_gemm_skinny_ranges": [P, I, L, P, I, I, I, P, L, I, I, I, P, L, P, I, P],
     },

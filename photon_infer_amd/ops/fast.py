@@ -217,7 +217,7 @@ def ranges_product_ok(tokens: int, head_dim: int, weight_bytes: int = 0) -> bool
 def merge_ranges(out: torch.Tensor, kr: KeyRanges) -> None:
     """The merged attention output, bfloat16 [tokens, heads * head_dim], by the merging kernel."""
     _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), kr.rows.data_ptr(), kr.tokens,
-              kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count, _stream())
+              kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count, None, None, _stream())
 
 
 def gemm_from_ranges(out, kr: KeyRanges, w, accumulate, N, ldw, ldc, may_defer, ws: Optional[KernelWorkspace]) -> bool:
@@ -499,7 +499,10 @@ def _decode_splits_that_fit(ws, n_req: int, num_heads: int, num_kv_heads: int, h
 
 
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                    page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None) -> bool:
+                    page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None, slopes=None, sinks=None, gate=None) -> bool:
+    """``slopes`` / ``sinks`` (float32 [heads]) and ``gate`` (float32 [tokens, heads]): a distance bias, a sink in
+    the softmax and an output gate per head (None: none)."""
+    opt = tuple(None if t is None else t.data_ptr() for t in (slopes, sinks, gate))
     if head_dim not in DECODE_HEAD_DIMS or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
         return False
     G = num_heads // num_kv_heads
@@ -511,7 +514,7 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
         _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
                   k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
                   ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), req_ids, n_req, num_heads, num_kv_heads, head_dim,
-                  page_size, float(scale), int(window), pages, splits, part.data_ptr(), part.numel(), _stream())
+                  page_size, float(scale), int(window), pages, splits, part.data_ptr(), part.numel(), *opt, _stream())
 
     if ctx.all_decode and G <= 16:
         decode_kernel(R, 0, ctx.max_kv_len)
@@ -531,10 +534,10 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
               k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
               ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), plan.req.data_ptr(), plan.q0.data_ptr(), plan.cut.data_ptr(),
               plan.z0.data_ptr(), tile_part.data_ptr(), plan.order.data_ptr(), plan.rounds, plan.seats, num_heads,
-              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, *opt, _stream())
     if plan.cut_tokens:
         _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), plan.rows.data_ptr(), plan.cut_tokens,
-                  tile_part.data_ptr(), num_heads, head_dim, plan.cuts, _stream())
+                  tile_part.data_ptr(), num_heads, head_dim, plan.cuts, opt[1], opt[2], _stream())
     return True
 
 

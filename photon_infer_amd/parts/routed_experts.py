@@ -20,6 +20,7 @@ from .. import ops
 from ..errors import UnsupportedModelError
 from ..weights.loader import TensorSpec
 from .base import FEED_FORWARDS, FeedForward, StepContext
+from .mlp import INTERLEAVE
 
 
 class RoutedExperts(FeedForward):
@@ -53,10 +54,20 @@ class RoutedExperts(FeedForward):
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
         E, p = self.num_experts, self.expert_prefix
-        # per expert [gate rows | up rows], stacked: [E, 2F, D]; down: [E, D, F]
-        self.w_gate_up = torch.stack([torch.cat([tensors[f"{p}{e}.{self.names[0]}"], tensors[f"{p}{e}.{self.names[1]}"]], dim=0)
-                                      for e in range(E)]).contiguous()
-        self.w_down = torch.stack([tensors[f"{p}{e}.{self.names[2]}"] for e in range(E)]).contiguous()
+        F, b = self.expert_size, INTERLEAVE
+        mats = []
+        for e in range(E):
+            g, u = tensors[f"{p}{e}.{self.names[0]}"], tensors[f"{p}{e}.{self.names[1]}"]
+            if g.dtype == torch.bfloat16 and u.dtype == torch.bfloat16 and F % b == 0:
+                # gate and up rows interleaved in blocks of 16, as the dense gated feed-forward keeps them: the
+                # matrix-core product then applies the activation before anything is stored
+                mats.append(torch.stack([g.view(F // b, b, -1), u.view(F // b, b, -1)], dim=1).reshape(2 * F, -1))
+            else:
+                mats.append(torch.cat([g, u], dim=0))
+        self.interleave = b if all(t.dtype == torch.bfloat16 for t in mats) and F % b == 0 else 0
+        self.w_gate_up = torch.stack(mats).contiguous()                   # [E, 2F, D]
+        self.w_down = torch.stack([tensors[f"{p}{e}.{self.names[2]}"] for e in range(E)]).contiguous()   # [E, D, F]
+        self.tile = ops.grouped_tile_rows(self.w_gate_up.dtype if self.w_down.dtype == self.w_gate_up.dtype else torch.float32)
         self.w_router = tensors[self.router_name]
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
@@ -64,12 +75,10 @@ class RoutedExperts(FeedForward):
         logits = torch.empty((T, self.num_experts), dtype=torch.float32, device=h.device)
         ops.gemm(logits, h, self.w_router, ws=ws)
         ids, weights = ops.route(logits, self.top, self.groups, self.keep, self.renormalize)
-        rows = ops.group_entries(ids, self.num_experts)
+        rows = ops.group_entries(ids, self.num_experts, self.tile)
         a = ops.gather_rows(h, rows)
-        gu = torch.empty((rows.rows, 2 * self.expert_size), dtype=self.dtype, device=h.device)
-        ops.grouped_gemm(gu, a, self.w_gate_up, rows)
         act = torch.empty((rows.rows, self.expert_size), dtype=self.dtype, device=h.device)
-        ops.swiglu(act, gu, 0)
+        ops.grouped_gemm_swiglu(act, a, self.w_gate_up, rows, self.interleave)
         y = torch.empty((rows.rows, self.hidden_size), dtype=torch.float32, device=h.device)
         ops.grouped_gemm(y, act, self.w_down, rows)
         if self.accumulate:

@@ -35,6 +35,7 @@ class PagedKV:
 
     def __init__(self, seqs: Sequence[tuple], page_size: int, dtype, seed: int = 0, spare_pages: int = 3):
         nkv, hd = seqs[0][0].shape[1:]
+        vd = seqs[0][1].shape[2]          # values may have another width than keys
         blocks = [-(-k.shape[0] // page_size) for k, _ in seqs]
         total = sum(blocks) + spare_pages
         g = torch.Generator().manual_seed(seed)
@@ -43,7 +44,7 @@ class PagedKV:
         self.table = torch.full((len(seqs), width), -1, dtype=torch.int32)
         # unused pages hold large values: a read outside a request's keys shows
         self.k = torch.full((total, nkv, page_size, hd), 1e4, dtype=torch.float32)
-        self.v = torch.full((total, nkv, hd, page_size), -1e4, dtype=torch.float32)   # values are kept transposed
+        self.v = torch.full((total, nkv, vd, page_size), -1e4, dtype=torch.float32)   # values are kept transposed
         it = iter(order)
         for r, (k, v) in enumerate(seqs):
             for b in range(blocks[r]):
