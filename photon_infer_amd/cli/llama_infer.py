@@ -114,9 +114,10 @@ def main(argv=None) -> int:
             max_step_tokens=args.max_step_tokens, chunk_size=args.chunk_size, max_model_len=args.max_model_len,
             seed=args.seed, max_cache_tokens=None if args.num_blocks else 65536)
         engine = ContinuousBatchEngine(model_dir, options)
-        cfg = engine.config
-        print(f"  Layers: {cfg.num_hidden_layers}")
-        print(f"  Dimension: {cfg.hidden_size}\n")
+        spec = engine.runner.spec           # any registered architecture: the model as data, not a config's field names
+        print(f"  Architecture: {engine.config.architecture}")
+        print(f"  Layers: {len(spec.layers)}")
+        print(f"  Dimension: {spec.hidden_size}\n")
         print("Model ready!\n")
         prompts = _prompts(args, tok)
         start = time.perf_counter()

@@ -12,7 +12,8 @@
 // result for a token does not depend on how the tokens were cut into steps.
 //
 // One wave per (request, head, 16 value columns): lane = column + 16 * part; the four parts split
-// the d rows of the state, which stays in registers over all tokens of the step.  n and m are kept
+// the d rows of the state, which stays in registers over all tokens of the step (rows beyond d are
+// zeros that never leave the registers).  n and m are kept
 // once per group of 16 columns ([slices, d + 1] per head), so that no block reads what another writes.
 //
 // State row of one request (floats): [heads][d][dv] S, then [heads][slices][d + 1] (n, then m).
@@ -28,60 +29,175 @@ __host__ __device__ inline long mm_state_floats(int heads, int d, int dv) {
 
 extern "C" long pi_matrix_memory_state_floats(int heads, int d, int dv) { return mm_state_floats(heads, d, dv); }
 
-template <int DPP>
+// Tokens are staged through LDS a chunk at a time (one trip to memory per chunk instead of one
+// per token).  Everything of a chunk that does not depend on the state is made before its walk:
+// the gates (lane j, token j), the running maximum (a short sequential pass over the chunk's
+// gates, the same in every lane) and from it each token's decay a, input weight b and floor
+// exp(-m).  The walk itself is multiply-adds on registers and LDS reads.
+//
+// Long portions are cut into segments of MM_SEGMENT tokens that run side by side.  The state's
+// recurrence is linear once a, b are known, and those depend on the gates alone:
+//   1. a gates kernel (one wave per request and head) makes a, b, exp(-m) for every token;
+//   2. every segment is walked from a zero state, leaving its summary (its own contribution L
+//      and the product A of its decays);
+//   3. every segment is walked again for its outputs, from the state at its start, which it gets
+//      by folding the summaries of the segments before it onto the request's state:
+//      S <- A S + L, segment by segment;
+//   4. a last kernel folds all summaries onto the request's state and stores it.
+// A step whose requests bring at most one segment each (decoding, short portions) is one kernel,
+// which makes its own gates.
+#define MM_SEGMENT 128
+
+// floats of one segment summary for one (head, column group): L's part of S [d][16], of n [d], then A
+__host__ __device__ inline long mm_summary_floats(int d) { return (long)d * MM_COLS + d + 1; }
+
+enum { MM_SINGLE = 0, MM_SUMMARY = 1, MM_OUTPUT = 2 };
+
+template <int DPP, int MODE>
 __global__ __launch_bounds__(PI_WAVE) void matrix_memory_scan_kernel(
     float* __restrict__ out, long out_stride, const float* __restrict__ proj, long proj_stride, int q_off, int k_off, int v_off,
     int i_off, int f_off, const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
     const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ state, long state_stride, int max_slots,
-    int heads, int d, int dv) {
-  const int r = blockIdx.x, h = blockIdx.y, slice = blockIdx.z;
+    int heads, int d, int dv, int segs, const float* __restrict__ coef, float* __restrict__ summaries) {
+  constexpr int DP = MM_PARTS * DPP;             // rows of the state as the lanes hold them (>= d)
+  constexpr int CH = 2048 / DP < PI_WAVE ? 2048 / DP : PI_WAVE;   // tokens per chunk: 8 KB of queries, as much of keys
+  __shared__ __attribute__((aligned(16))) float qs[CH][DP];
+  __shared__ __attribute__((aligned(16))) float ks[CH][DP];
+  __shared__ float vs[CH][MM_COLS];
+  __shared__ float gi[CH], gf[CH], wa[CH], wb[CH], we[CH];
+  const int r = blockIdx.x / segs, seg = blockIdx.x % segs, h = blockIdx.y, slice = blockIdx.z;
   const int lane = threadIdx.x, col = lane % MM_COLS, part = lane / MM_COLS;
   const int c = slice * MM_COLS + col;
   const bool col_ok = c < dv;
   const int slot = slots[r];
   if (slot < 0 || slot >= max_slots) return;
   const int slices = gridDim.z;
+  const int t0 = MODE == MM_SINGLE ? q_start[r] : q_start[r] + seg * MM_SEGMENT;
+  const int t1 = MODE == MM_SINGLE ? q_start[r + 1] : min(q_start[r + 1], t0 + MM_SEGMENT);
+  if (t0 >= t1) return;                          // the request has fewer segments
   float* Sg = state + (long)slot * state_stride + (long)h * d * dv;
   float* nm = state + (long)slot * state_stride + (long)heads * d * dv + ((long)h * slices + slice) * (d + 1);
+  const long sum_floats = mm_summary_floats(d);
+  float* sums = MODE == MM_SINGLE ? nullptr : summaries + (((long)r * segs * heads + h) * slices + slice) * sum_floats;
+  const long sum_stride = (long)heads * slices * sum_floats;      // from one segment's summary to the next
   const int r0 = part * DPP;                     // this lane's rows of the state: r0 .. r0 + DPP - 1 (those below d)
   float S[DPP], n[DPP];
 #pragma unroll
   for (int i = 0; i < DPP; ++i) {
     const bool ok = r0 + i < d;
-    S[i] = (ok && col_ok) ? Sg[(long)(r0 + i) * dv + c] : 0.f;
-    n[i] = ok ? nm[r0 + i] : 0.f;
+    S[i] = (MODE != MM_SUMMARY && ok && col_ok) ? Sg[(long)(r0 + i) * dv + c] : 0.f;
+    n[i] = (MODE != MM_SUMMARY && ok) ? nm[r0 + i] : 0.f;
   }
-  float m = nm[d];
-  const int t0 = q_start[r], t1 = q_start[r + 1];
-  for (int t = t0; t < t1; ++t) {
-    const float* row = proj + (long)t * proj_stride;
-    const float zi = row[i_off + h] + i_bias[h], zf = row[f_off + h] + f_bias[h];
-    const float ig = cap * tanhf(zi / cap);
-    const float fz = cap * tanhf(zf / cap);
-    const float fg = fminf(fz, 0.f) - log1pf(expf(-fabsf(fz)));
-    const float m_new = fmaxf(fg + m, ig);
-    const float a = expf(fg + m - m_new), b = expf(ig - m_new);
-    const float v = col_ok ? row[v_off + h * dv + c] : 0.f;
-    const float bv = b * v;
-    const float* qr = row + q_off + h * d + r0;
-    const float* kr = row + k_off + h * d + r0;
-    float num = 0.f, den = 0.f;
+  if (MODE == MM_OUTPUT) {                       // the state at the segment's start
+    for (int s = 0; s < seg; ++s) {
+      const float* L = sums + s * sum_stride;
+      const float A = L[sum_floats - 1];
+#pragma unroll
+      for (int i = 0; i < DPP; ++i) {
+        if (r0 + i < d) {
+          S[i] = fmaf(A, S[i], L[(r0 + i) * MM_COLS + col]);
+          n[i] = fmaf(A, n[i], L[d * MM_COLS + r0 + i]);
+        }
+      }
+    }
+  }
+  float m = MODE == MM_SINGLE ? nm[d] : 0.f;
+  float decay = 1.0f;                            // MM_SUMMARY: the product of the segment's decays
+  const float bi = i_bias[h], bf = f_bias[h];
+  for (int tc = t0; tc < t1; tc += CH) {
+    const int nt = min(CH, t1 - tc);
+    // the chunk's queries (scaled), keys and this block's value columns; rows beyond d are zero
+    for (int idx = lane; idx < nt * DP; idx += PI_WAVE) {
+      const int j = idx / DP, i = idx % DP;
+      const float* row = proj + (long)(tc + j) * proj_stride;
+      if (MODE != MM_SUMMARY) qs[j][i] = i < d ? row[q_off + h * d + i] * q_scale : 0.f;
+      ks[j][i] = i < d ? row[k_off + h * d + i] : 0.f;
+    }
+    for (int idx = lane; idx < nt * MM_COLS; idx += PI_WAVE) {
+      const int j = idx / MM_COLS, cc = slice * MM_COLS + idx % MM_COLS;
+      vs[j][idx % MM_COLS] = cc < dv ? proj[(long)(tc + j) * proj_stride + v_off + h * dv + cc] : 0.f;
+    }
+    if (MODE == MM_SINGLE) {
+      if (lane < nt) {
+        const float* row = proj + (long)(tc + lane) * proj_stride;
+        const float fz = cap * tanhf((row[f_off + h] + bf) / cap);
+        gi[lane] = cap * tanhf((row[i_off + h] + bi) / cap);
+        gf[lane] = fminf(fz, 0.f) - log1pf(expf(-fabsf(fz)));
+      }
+      __syncthreads();
+      // the running maximum over the chunk (every lane the same); lane j keeps token j's
+      float m_before = m, m_mine = m;
+      for (int j = 0; j < nt; ++j) {
+        const float m_new = fmaxf(gf[j] + m, gi[j]);
+        if (j == lane) {
+          m_before = m;
+          m_mine = m_new;
+        }
+        m = m_new;
+      }
+      if (lane < nt) {
+        wa[lane] = expf(gf[lane] + m_before - m_mine);
+        wb[lane] = expf(gi[lane] - m_mine);
+        we[lane] = expf(-m_mine);
+      }
+    } else if (lane < nt) {
+      const float* cf = coef + ((long)(tc + lane) * heads + h) * 3;
+      wa[lane] = cf[0];
+      wb[lane] = cf[1];
+      we[lane] = cf[2];
+    }
+    __syncthreads();
+    for (int j = 0; j < nt; ++j) {
+      const float a = wa[j], b = wb[j];
+      const float bv = b * vs[j][col];
+      float num[4] = {0.f, 0.f, 0.f, 0.f}, den[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < DPP; i += 4) {
+        const float4 kk = *reinterpret_cast<const float4*>(&ks[j][r0 + i]);
+        const float kv[4] = {kk.x, kk.y, kk.z, kk.w};
+        if (MODE == MM_SUMMARY) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            S[i + u] = fmaf(a, S[i + u], kv[u] * bv);
+            n[i + u] = fmaf(a, n[i + u], b * kv[u]);
+          }
+        } else {
+          const float4 qq = *reinterpret_cast<const float4*>(&qs[j][r0 + i]);
+          const float qv[4] = {qq.x, qq.y, qq.z, qq.w};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            S[i + u] = fmaf(a, S[i + u], kv[u] * bv);
+            n[i + u] = fmaf(a, n[i + u], b * kv[u]);
+            num[u] = fmaf(S[i + u], qv[u], num[u]);
+            den[u] = fmaf(n[i + u], qv[u], den[u]);
+          }
+        }
+      }
+      if (MODE == MM_SUMMARY) {
+        decay *= a;
+      } else {
+        float nu = (num[0] + num[1]) + (num[2] + num[3]), de = (den[0] + den[1]) + (den[2] + den[3]);
+        nu += __shfl_xor(nu, 16, PI_WAVE);
+        de += __shfl_xor(de, 16, PI_WAVE);
+        nu += __shfl_xor(nu, 32, PI_WAVE);
+        de += __shfl_xor(de, 32, PI_WAVE);
+        if (part == 0 && col_ok) out[(long)(tc + j) * out_stride + h * dv + c] = nu / (fmaxf(fabsf(de), we[j]) + 1e-6f);
+      }
+    }
+    __syncthreads();
+  }
+  if (MODE == MM_OUTPUT) return;                 // the state is stored by the folding kernel
+  if (MODE == MM_SUMMARY) {
+    float* L = sums + seg * sum_stride;
 #pragma unroll
     for (int i = 0; i < DPP; ++i) {
       if (r0 + i < d) {
-        const float kk = kr[i], qq = qr[i] * q_scale;
-        S[i] = fmaf(a, S[i], kk * bv);
-        n[i] = fmaf(a, n[i], b * kk);
-        num = fmaf(S[i], qq, num);
-        den = fmaf(n[i], qq, den);
+        L[(r0 + i) * MM_COLS + col] = S[i];
+        if (col == 0) L[d * MM_COLS + r0 + i] = n[i];
       }
     }
-    num += __shfl_xor(num, 16, PI_WAVE);
-    den += __shfl_xor(den, 16, PI_WAVE);
-    num += __shfl_xor(num, 32, PI_WAVE);
-    den += __shfl_xor(den, 32, PI_WAVE);
-    m = m_new;
-    if (part == 0 && col_ok) out[(long)t * out_stride + h * dv + c] = num / (fmaxf(fabsf(den), expf(-m_new)) + 1e-6f);
+    if (lane == 0) L[sum_floats - 1] = decay;
+    return;
   }
 #pragma unroll
   for (int i = 0; i < DPP; ++i) {
@@ -93,14 +209,93 @@ __global__ __launch_bounds__(PI_WAVE) void matrix_memory_scan_kernel(
   if (lane == 0) nm[d] = m;
 }
 
+// a, b and exp(-m) of every token of the step, [T, heads, 3], and the running maximum after each
+// request's last token, [R, heads].  One wave per (request, head): 64 tokens' gates at a time
+// (lane j, token j), then the maximum's chain over them, handed round by lane shuffles.
+__global__ __launch_bounds__(PI_WAVE) void matrix_memory_gates_kernel(
+    float* __restrict__ coef, float* __restrict__ m_end, const float* __restrict__ proj, long proj_stride, int i_off, int f_off,
+    const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, const int* __restrict__ q_start,
+    const int* __restrict__ slots, const float* __restrict__ state, long state_stride, int max_slots, int heads, int d, int dv) {
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int slot = slots[r];
+  if (slot < 0 || slot >= max_slots) return;
+  const int slices = (dv + MM_COLS - 1) / MM_COLS;
+  float m = state[(long)slot * state_stride + (long)heads * d * dv + ((long)h * slices) * (d + 1) + d];
+  const float bi = i_bias[h], bf = f_bias[h];
+  const int t0 = q_start[r], t1 = q_start[r + 1];
+  for (int tc = t0; tc < t1; tc += PI_WAVE) {
+    const int nt = min(PI_WAVE, t1 - tc);
+    float gi = 0.f, gf = 0.f;
+    if (lane < nt) {
+      const float* row = proj + (long)(tc + lane) * proj_stride;
+      const float fz = cap * tanhf((row[f_off + h] + bf) / cap);
+      gi = cap * tanhf((row[i_off + h] + bi) / cap);
+      gf = fminf(fz, 0.f) - log1pf(expf(-fabsf(fz)));
+    }
+    float m_before = m, m_mine = m;
+    for (int j = 0; j < nt; ++j) {
+      const float m_new = fmaxf(__shfl(gf, j, PI_WAVE) + m, __shfl(gi, j, PI_WAVE));
+      if (j == lane) {
+        m_before = m;
+        m_mine = m_new;
+      }
+      m = m_new;
+    }
+    if (lane < nt) {
+      float* cf = coef + ((long)(tc + lane) * heads + h) * 3;
+      cf[0] = expf(gf + m_before - m_mine);
+      cf[1] = expf(gi - m_mine);
+      cf[2] = expf(-m_mine);
+    }
+  }
+  if (lane == 0) m_end[r * heads + h] = m;
+}
+
+// The request's state after the step: all its segments' summaries folded onto the old state.
+__global__ __launch_bounds__(256) void matrix_memory_fold_kernel(float* __restrict__ state, long state_stride, int max_slots,
+                                                                 const int* __restrict__ q_start, const int* __restrict__ slots,
+                                                                 const float* __restrict__ summaries, const float* __restrict__ m_end,
+                                                                 int heads, int d, int dv, int segs) {
+  const int r = blockIdx.x, h = blockIdx.y, slice = blockIdx.z, slices = gridDim.z;
+  const int slot = slots[r];
+  if (slot < 0 || slot >= max_slots) return;
+  const int n_seg = (q_start[r + 1] - q_start[r] + MM_SEGMENT - 1) / MM_SEGMENT;
+  float* Sg = state + (long)slot * state_stride + (long)h * d * dv;
+  float* nm = state + (long)slot * state_stride + (long)heads * d * dv + ((long)h * slices + slice) * (d + 1);
+  const long sum_floats = mm_summary_floats(d);
+  const float* sums = summaries + (((long)r * segs * heads + h) * slices + slice) * sum_floats;
+  const long sum_stride = (long)heads * slices * sum_floats;
+  for (int idx = threadIdx.x; idx < d * MM_COLS + d; idx += blockDim.x) {
+    const bool is_n = idx >= d * MM_COLS;
+    const int row = is_n ? idx - d * MM_COLS : idx / MM_COLS, c = slice * MM_COLS + idx % MM_COLS;
+    if (!is_n && c >= dv) continue;
+    float* where = is_n ? nm + row : Sg + (long)row * dv + c;
+    float v = *where;
+    for (int s = 0; s < n_seg; ++s) v = fmaf(sums[s * sum_stride + sum_floats - 1], v, sums[s * sum_stride + idx]);
+    *where = v;
+  }
+  if (threadIdx.x == 0) nm[d] = m_end[r * heads + h];
+}
+
+extern "C" int pi_matrix_memory_segment() { return MM_SEGMENT; }
+
 // out float32 [T, heads * dv]: the cell's raw output per head.  proj float32 rows hold q, k
 // ([heads, d] each), v ([heads, dv]) and the gate pre-activations ([heads] each) at the given
 // column offsets.  Requests r = 0 .. R-1 own tokens q_start[r] .. q_start[r+1]; their states are
-// rows slots[r] of `state`.
+// rows slots[r] of `state`.  max_q_len: the most tokens a request brings (an upper bound will do);
+// above MM_SEGMENT the step runs in segments and needs `work`: float32, at least
+// pi_matrix_memory_work_floats(T, R, max_q_len, heads, d, dv).
+extern "C" long pi_matrix_memory_work_floats(int T, int R, int max_q_len, int heads, int d, int dv) {
+  if (max_q_len <= MM_SEGMENT) return 0;
+  const long segs = (max_q_len + MM_SEGMENT - 1) / MM_SEGMENT, slices = (dv + MM_COLS - 1) / MM_COLS;
+  return (long)T * heads * 3 + (long)R * heads + (long)R * segs * heads * slices * mm_summary_floats(d);
+}
+
 extern "C" int pi_matrix_memory_scan(float* out, long out_stride, const float* proj, long proj_stride, int q_off, int k_off,
                                      int v_off, int i_off, int f_off, const float* i_bias, const float* f_bias, float cap,
                                      float q_scale, const int* q_start, const int* slots, int R, float* state,
-                                     long state_stride, int max_slots, int heads, int d, int dv, hipStream_t stream) {
+                                     long state_stride, int max_slots, int heads, int d, int dv, int T, int max_q_len,
+                                     float* work, long work_floats, hipStream_t stream) {
   PI_REQUIRE(R >= 0 && heads > 0 && d > 0 && dv > 0, "matrix memory: bad sizes");
   PI_REQUIRE(d <= 4 * 64, "matrix memory: key size %d is above %d", d, 4 * 64);
   PI_REQUIRE(state_stride >= mm_state_floats(heads, d, dv), "matrix memory: state rows of %ld floats are too short", state_stride);
@@ -109,15 +304,36 @@ extern "C" int pi_matrix_memory_scan(float* out, long out_stride, const float* p
   if (R == 0) return 0;
   const int slices = (dv + MM_COLS - 1) / MM_COLS;
   PI_REQUIRE(slices <= 65535, "matrix memory: value size %d is too large", dv);
-  const dim3 grid(R, heads, slices), block(PI_WAVE);
+  const int segs = max_q_len <= MM_SEGMENT ? 1 : (max_q_len + MM_SEGMENT - 1) / MM_SEGMENT;
+  PI_REQUIRE((long)R * segs < 2147483647L, "matrix memory: too many segments");
+  PI_REQUIRE(segs == 1 || (work && work_floats >= pi_matrix_memory_work_floats(T, R, max_q_len, heads, d, dv)),
+             "matrix memory: a step in %d segments needs its workspace", segs);
+  float* coef = work;
+  float* m_end = segs > 1 ? coef + (long)T * heads * 3 : nullptr;
+  float* summaries = segs > 1 ? m_end + (long)R * heads : nullptr;
+  const dim3 grid(R * segs, heads, slices), block(PI_WAVE);
   const int dpp = (d + MM_PARTS - 1) / MM_PARTS;
-#define MM_GO(DPP) hipLaunchKernelGGL(matrix_memory_scan_kernel<DPP>, grid, block, 0, stream, out, out_stride, proj, proj_stride, q_off, \
+#define MM_GO(DPP, MODE) hipLaunchKernelGGL((matrix_memory_scan_kernel<DPP, MODE>), grid, block, 0, stream, out, out_stride, proj, proj_stride, q_off, \
                                       k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, q_start, slots, state, state_stride,    \
-                                      max_slots, heads, d, dv)
-  if (dpp <= 8) MM_GO(8);
-  else if (dpp <= 16) MM_GO(16);
-  else if (dpp <= 32) MM_GO(32);
-  else MM_GO(64);
+                                      max_slots, heads, d, dv, segs, coef, summaries)
+#define MM_PICK(MODE)                \
+  do {                               \
+    if (dpp <= 8) MM_GO(8, MODE);    \
+    else if (dpp <= 16) MM_GO(16, MODE); \
+    else if (dpp <= 32) MM_GO(32, MODE); \
+    else MM_GO(64, MODE);            \
+  } while (0)
+  if (segs == 1) {
+    MM_PICK(MM_SINGLE);
+    return pi_check_launch("matrix_memory_scan");
+  }
+  hipLaunchKernelGGL(matrix_memory_gates_kernel, dim3(R, heads), block, 0, stream, coef, m_end, proj, proj_stride, i_off, f_off, i_bias,
+                     f_bias, cap, q_start, slots, state, state_stride, max_slots, heads, d, dv);
+  MM_PICK(MM_SUMMARY);
+  MM_PICK(MM_OUTPUT);
+  hipLaunchKernelGGL(matrix_memory_fold_kernel, dim3(R, heads, slices), dim3(256), 0, stream, state, state_stride, max_slots, q_start,
+                     slots, summaries, m_end, heads, d, dv, segs);
+#undef MM_PICK
 #undef MM_GO
   return pi_check_launch("matrix_memory_scan");
 }

@@ -11,6 +11,7 @@ goes to the general kernels (module "core"), which take any size.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -596,10 +597,18 @@ def matrix_memory_scan(out: torch.Tensor, proj: torch.Tensor, offsets, i_bias: t
         raise KernelError(f"matrix memory: state must be contiguous float32 [slots, >= {floats}], got {state.dtype} {tuple(state.shape)}")
     _i32(ctx.q_start, "q_start", ctx.R + 1)
     _i32(ctx.slots, "slots", ctx.R)
+    # a request that brings more than one segment of tokens is walked in segments side by side, which
+    # needs scratch memory; the most tokens of a request is a host-side number of the step (1 in a
+    # step of single tokens, so a replayed decode step never takes this path)
+    longest = int(getattr(ctx, "max_q_len", 0) or T)
+    lib = _lib.load("core")
+    lib.pi_matrix_memory_work_floats.restype = ctypes.c_long
+    floats = int(lib.pi_matrix_memory_work_floats(T, ctx.R, longest, heads, key_dim, value_dim))
+    work = torch.empty(floats, dtype=torch.float32, device=out.device) if floats else None
     _lib.call("core", "pi_matrix_memory_scan", out.data_ptr(), _rows(out, "out"), proj.data_ptr(), _rows(proj, "projection"),
               int(offsets[0]), int(offsets[1]), int(offsets[2]), int(offsets[3]), int(offsets[4]), i_bias.data_ptr(),
               f_bias.data_ptr(), float(cap), float(q_scale), ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R,
-              state.data_ptr(), state.shape[1], state.shape[0], heads, key_dim, value_dim, _stream())
+              state.data_ptr(), state.shape[1], state.shape[0], heads, key_dim, value_dim, T, longest, _ptr(work), floats, _stream())
 
 
 def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, value_dim: int) -> None:

@@ -24,7 +24,7 @@ _SIGNATURES = {
         "pi_branch_norm_add": [P, P, I, P, P, P, P, P, F, F, I, I, P],
         "pi_cast_stream": [P, I, P, L, P],
         "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P],
-        "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, P],
+        "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, I, I, P, L, P],
         "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, P],
         "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
         "pi_group_entries": [P, I, I, P, P, P, P, P, I, I, P],

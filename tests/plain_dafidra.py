@@ -4,7 +4,7 @@ float64.  It shares no code with ``photon_infer_amd`` and reads a model folder b
 
 Notation: T tokens at positions 0 .. T-1, h [T, D] a sublayer's input, rows of weight matrices
 are outputs (y = W h).  ``act_round`` (optional) rounds activations where a bfloat16 engine
-rounds them (a sublayer's input, the attention's queries / keys / values and output, the
+rounds them (a sublayer's input, the attention's queries / keys / values, weights and output, the
 memory's output before its projection, the gated product), which gives tests a yardstick for
 the bfloat16 path; None rounds nothing.
 """
@@ -73,6 +73,8 @@ def sink_window_attention(h: torch.Tensor, W: Dict[str, torch.Tensor], c: dict, 
             scores = [float(q[i, n * d:(n + 1) * d] @ k[j, g * d:(g + 1) * d]) * c["scale"] - distance_slope(n, H) * (i - j)
                       for j in range(lo, i + 1)]
             probs = sink_softmax(scores, float(W["sink"][n]))
+            if act_round is not None:      # a bfloat16 engine may round the weights for their product with the values
+                probs = _r(torch.tensor(probs, dtype=F), act_round).tolist()
             acc = torch.zeros(dv, dtype=F)
             for j, p in zip(range(lo, i + 1), probs):
                 acc += p * v[j, g * dv:(g + 1) * dv]
@@ -110,7 +112,7 @@ def matrix_memory(h: torch.Tensor, W: Dict[str, torch.Tensor], c: dict, eps: flo
 
 
 def gated_ffn(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, act_round: Round = None) -> torch.Tensor:
-    g, u = h @ gate.T, h @ up.T
+    g, u = _r(h @ gate.T, act_round), _r(h @ up.T, act_round)       # a bfloat16 engine may store the two products before it gates
     return _r(g * torch.sigmoid(g) * u, act_round) @ down.T
 
 
@@ -142,7 +144,11 @@ def route_margin(z: torch.Tensor, top: int, groups: int, keep: int) -> float:
     return margin
 
 
-def routed_experts(h: torch.Tensor, W: Dict[str, torch.Tensor], c: dict, act_round: Round = None, margins: Optional[list] = None) -> torch.Tensor:
+def routed_experts(h: torch.Tensor, W: Dict[str, torch.Tensor], c: dict, act_round: Round = None, margins: Optional[list] = None,
+                   forced=None, chosen: Optional[list] = None) -> torch.Tensor:
+    """``forced`` ([T, top] expert ids): use these experts instead of the router's own choice, each with its own
+    score (for comparisons with an engine whose rounding decided a close call the other way); ``chosen`` receives
+    the router's own choice per token."""
     r = c["router"]
     g = r.get("groups") or {"count": 1, "keep": 1}
     out = torch.zeros_like(h)
@@ -150,7 +156,13 @@ def routed_experts(h: torch.Tensor, W: Dict[str, torch.Tensor], c: dict, act_rou
     for t in range(h.shape[0]):
         if margins is not None:
             margins.append(route_margin(z[t], r["top"], g["count"], g["keep"]))
-        for e, w in route(z[t], r["top"], g["count"], g["keep"]):
+        own = route(z[t], r["top"], g["count"], g["keep"])
+        if chosen is not None:
+            chosen.append([e for e, _ in own])
+        if forced is not None:
+            s = torch.softmax(z[t], dim=-1)
+            own = [(int(e), float(s[int(e)])) for e in forced[t]]
+        for e, w in own:
             out[t] += w * gated_ffn(h[t:t + 1], W[f"e{e}.gate"], W[f"e{e}.up"], W[f"e{e}.down"], act_round)[0]
     return out
 
@@ -160,9 +172,10 @@ def _sub(tensors: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tenso
 
 
 def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], act_round: Round = None, streams: Optional[list] = None,
-            margins: Optional[list] = None):
+            margins: Optional[list] = None, forced: Optional[dict] = None, chosen: Optional[dict] = None):
     """float64 logits [T, vocab] of a whole sequence; ``streams`` (a list) receives the residual stream after every layer,
-    ``margins`` (a list) every routing decision's margin (``route_margin``)."""
+    ``margins`` (a list) every routing decision's margin (``route_margin``); ``forced`` / ``chosen``: per routed layer
+    (by layer index) the experts to use / the router's own choices, see ``routed_experts``."""
     eps, m = config["norm"]["eps"], config["residual_mult"]
     x = torch.stack([tensors["embed"][int(t)].to(F) for t in tokens])
     for i, layer in enumerate(config["layers"]):
@@ -176,7 +189,9 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], a
         if layer["mlp"] is not None:
             h = _r(x, act_round)
             W = _sub(tensors, p + "mlp.")
-            f = gated_ffn(h, W["gate"], W["up"], W["down"], act_round) if layer["mlp"]["kind"] == "dense" else routed_experts(h, W, layer["mlp"], act_round, margins)
+            f = gated_ffn(h, W["gate"], W["up"], W["down"], act_round) if layer["mlp"]["kind"] == "dense" else routed_experts(
+                h, W, layer["mlp"], act_round, margins if margins is None else margins.setdefault(i, []) if isinstance(margins, dict) else margins,
+                forced.get(i) if forced else None, chosen.setdefault(i, []) if chosen is not None else None)
             x = x + m * rms_norm(f, tensors[p + "norm2"].to(F), eps, 1.0)
         if streams is not None:
             streams.append(x.clone())
