@@ -35,18 +35,18 @@ extern "C" long pi_matrix_memory_state_floats(int heads, int d, int dv) { return
 // gates, the same in every lane) and from it each token's decay a, input weight b and floor
 // exp(-m).  The walk itself is multiply-adds on registers and LDS reads.
 //
-// Long portions are cut into segments of MM_SEGMENT tokens that run side by side.  The state's
+// Long portions are cut into segments of MM_SEGMENT tokens that run side by side (with 64 tokens a
+// 2,048-token prompt gives every SIMD of the chip four waves to switch between).  The state's
 // recurrence is linear once a, b are known, and those depend on the gates alone:
 //   1. a gates kernel (one wave per request and head) makes a, b, exp(-m) for every token;
 //   2. every segment is walked from a zero state, leaving its summary (its own contribution L
 //      and the product A of its decays);
-//   3. every segment is walked again for its outputs, from the state at its start, which it gets
-//      by folding the summaries of the segments before it onto the request's state:
-//      S <- A S + L, segment by segment;
-//   4. a last kernel folds all summaries onto the request's state and stores it.
+//   3. a prefix kernel turns the summaries into the states at the segments' starts (S <- A S + L,
+//      segment by segment, from the request's state) and stores the state after the step;
+//   4. every segment is walked again for its outputs, from the state at its start.
 // A step whose requests bring at most one segment each (decoding, short portions) is one kernel,
 // which makes its own gates.
-#define MM_SEGMENT 128
+#define MM_SEGMENT 64
 
 // floats of one segment summary for one (head, column group): L's part of S [d][16], of n [d], then A
 __host__ __device__ inline long mm_summary_floats(int d) { return (long)d * MM_COLS + d + 1; }
@@ -85,20 +85,16 @@ __global__ __launch_bounds__(PI_WAVE) void matrix_memory_scan_kernel(
 #pragma unroll
   for (int i = 0; i < DPP; ++i) {
     const bool ok = r0 + i < d;
-    S[i] = (MODE != MM_SUMMARY && ok && col_ok) ? Sg[(long)(r0 + i) * dv + c] : 0.f;
-    n[i] = (MODE != MM_SUMMARY && ok) ? nm[r0 + i] : 0.f;
+    S[i] = (MODE == MM_SINGLE && ok && col_ok) ? Sg[(long)(r0 + i) * dv + c] : 0.f;
+    n[i] = (MODE == MM_SINGLE && ok) ? nm[r0 + i] : 0.f;
   }
-  if (MODE == MM_OUTPUT) {                       // the state at the segment's start
-    for (int s = 0; s < seg; ++s) {
-      const float* L = sums + s * sum_stride;
-      const float A = L[sum_floats - 1];
+  if (MODE == MM_OUTPUT) {                       // the state at the segment's start, left by the prefix kernel in the summary's place
+    const float* L = sums + seg * sum_stride;
 #pragma unroll
-      for (int i = 0; i < DPP; ++i) {
-        if (r0 + i < d) {
-          S[i] = fmaf(A, S[i], L[(r0 + i) * MM_COLS + col]);
-          n[i] = fmaf(A, n[i], L[d * MM_COLS + r0 + i]);
-        }
-      }
+    for (int i = 0; i < DPP; ++i) {
+      const bool ok = r0 + i < d;
+      S[i] = ok ? L[(r0 + i) * MM_COLS + col] : 0.f;
+      n[i] = ok ? L[d * MM_COLS + r0 + i] : 0.f;
     }
   }
   float m = MODE == MM_SINGLE ? nm[d] : 0.f;
@@ -107,15 +103,38 @@ __global__ __launch_bounds__(PI_WAVE) void matrix_memory_scan_kernel(
   for (int tc = t0; tc < t1; tc += CH) {
     const int nt = min(CH, t1 - tc);
     // the chunk's queries (scaled), keys and this block's value columns; rows beyond d are zero
-    for (int idx = lane; idx < nt * DP; idx += PI_WAVE) {
-      const int j = idx / DP, i = idx % DP;
-      const float* row = proj + (long)(tc + j) * proj_stride;
-      if (MODE != MM_SUMMARY) qs[j][i] = i < d ? row[q_off + h * d + i] * q_scale : 0.f;
-      ks[j][i] = i < d ? row[k_off + h * d + i] : 0.f;
-    }
-    for (int idx = lane; idx < nt * MM_COLS; idx += PI_WAVE) {
-      const int j = idx / MM_COLS, cc = slice * MM_COLS + idx % MM_COLS;
-      vs[j][idx % MM_COLS] = cc < dv ? proj[(long)(tc + j) * proj_stride + v_off + h * dv + cc] : 0.f;
+    // (all loads of a chunk are asked for before the first is stored: one wait for memory per chunk)
+    {
+      constexpr int PER = CH * DP / PI_WAVE;     // elements of q, and of k, per lane: 32 whatever the sizes
+      float kreg[PER], qreg[PER];
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int idx = lane + u * PI_WAVE, j = idx / DP, i = idx % DP;
+        const bool in = j < nt && i < d;
+        const float* row = proj + (long)(tc + (in ? j : 0)) * proj_stride + h * d + (in ? i : 0);
+        kreg[u] = row[k_off];
+        if (MODE != MM_SUMMARY) qreg[u] = row[q_off];
+      }
+      constexpr int VPER = CH * MM_COLS / PI_WAVE;
+      float vreg[VPER];
+#pragma unroll
+      for (int u = 0; u < VPER; ++u) {
+        const int idx = lane + u * PI_WAVE, j = idx / MM_COLS, cc = slice * MM_COLS + idx % MM_COLS;
+        const bool in = j < nt && cc < dv;
+        vreg[u] = proj[(long)(tc + (in ? j : 0)) * proj_stride + v_off + h * dv + (in ? cc : 0)];
+      }
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int idx = lane + u * PI_WAVE, j = idx / DP, i = idx % DP;
+        const bool in = j < nt && i < d;
+        ks[j][i] = in ? kreg[u] : 0.f;
+        if (MODE != MM_SUMMARY) qs[j][i] = in ? qreg[u] * q_scale : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < VPER; ++u) {
+        const int idx = lane + u * PI_WAVE, j = idx / MM_COLS, cc = slice * MM_COLS + idx % MM_COLS;
+        vs[j][idx % MM_COLS] = (j < nt && cc < dv) ? vreg[u] : 0.f;
+      }
     }
     if (MODE == MM_SINGLE) {
       if (lane < nt) {
@@ -186,7 +205,7 @@ __global__ __launch_bounds__(PI_WAVE) void matrix_memory_scan_kernel(
     }
     __syncthreads();
   }
-  if (MODE == MM_OUTPUT) return;                 // the state is stored by the folding kernel
+  if (MODE == MM_OUTPUT) return;                 // the state was stored by the prefix kernel
   if (MODE == MM_SUMMARY) {
     float* L = sums + seg * sum_stride;
 #pragma unroll
@@ -210,52 +229,61 @@ __global__ __launch_bounds__(PI_WAVE) void matrix_memory_scan_kernel(
 }
 
 // a, b and exp(-m) of every token of the step, [T, heads, 3], and the running maximum after each
-// request's last token, [R, heads].  One wave per (request, head): 64 tokens' gates at a time
-// (lane j, token j), then the maximum's chain over them, handed round by lane shuffles.
-__global__ __launch_bounds__(PI_WAVE) void matrix_memory_gates_kernel(
+// request's last token, [R, heads].  One block per (request, head): 256 tokens' gates at a time
+// (thread j, token j) into LDS, then the maximum's chain over them (two operations per token, the
+// same in every thread, its LDS reads independent of the chain), then each thread its token's three numbers.
+#define MM_GATES_BLOCK 256
+__global__ __launch_bounds__(MM_GATES_BLOCK) void matrix_memory_gates_kernel(
     float* __restrict__ coef, float* __restrict__ m_end, const float* __restrict__ proj, long proj_stride, int i_off, int f_off,
     const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, const int* __restrict__ q_start,
     const int* __restrict__ slots, const float* __restrict__ state, long state_stride, int max_slots, int heads, int d, int dv) {
-  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  __shared__ float gis[MM_GATES_BLOCK], gfs[MM_GATES_BLOCK];
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int slot = slots[r];
   if (slot < 0 || slot >= max_slots) return;
   const int slices = (dv + MM_COLS - 1) / MM_COLS;
   float m = state[(long)slot * state_stride + (long)heads * d * dv + ((long)h * slices) * (d + 1) + d];
   const float bi = i_bias[h], bf = f_bias[h];
   const int t0 = q_start[r], t1 = q_start[r + 1];
-  for (int tc = t0; tc < t1; tc += PI_WAVE) {
-    const int nt = min(PI_WAVE, t1 - tc);
+  for (int tc = t0; tc < t1; tc += MM_GATES_BLOCK) {
+    const int nt = min(MM_GATES_BLOCK, t1 - tc);
     float gi = 0.f, gf = 0.f;
-    if (lane < nt) {
-      const float* row = proj + (long)(tc + lane) * proj_stride;
+    if (tid < nt) {
+      const float* row = proj + (long)(tc + tid) * proj_stride;
       const float fz = cap * tanhf((row[f_off + h] + bf) / cap);
       gi = cap * tanhf((row[i_off + h] + bi) / cap);
       gf = fminf(fz, 0.f) - log1pf(expf(-fabsf(fz)));
     }
+    __syncthreads();                 // the chain of the chunk before has been read
+    gis[tid] = gi;
+    gfs[tid] = gf;
+    __syncthreads();
     float m_before = m, m_mine = m;
     for (int j = 0; j < nt; ++j) {
-      const float m_new = fmaxf(__shfl(gf, j, PI_WAVE) + m, __shfl(gi, j, PI_WAVE));
-      if (j == lane) {
+      const float m_new = fmaxf(gfs[j] + m, gis[j]);
+      if (j == tid) {
         m_before = m;
         m_mine = m_new;
       }
       m = m_new;
     }
-    if (lane < nt) {
-      float* cf = coef + ((long)(tc + lane) * heads + h) * 3;
+    if (tid < nt) {
+      float* cf = coef + ((long)(tc + tid) * heads + h) * 3;
       cf[0] = expf(gf + m_before - m_mine);
       cf[1] = expf(gi - m_mine);
       cf[2] = expf(-m_mine);
     }
   }
-  if (lane == 0) m_end[r * heads + h] = m;
+  if (tid == 0) m_end[r * heads + h] = m;
 }
 
-// The request's state after the step: all its segments' summaries folded onto the old state.
-__global__ __launch_bounds__(256) void matrix_memory_fold_kernel(float* __restrict__ state, long state_stride, int max_slots,
-                                                                 const int* __restrict__ q_start, const int* __restrict__ slots,
-                                                                 const float* __restrict__ summaries, const float* __restrict__ m_end,
-                                                                 int heads, int d, int dv, int segs) {
+// From the segments' summaries to the states at their starts: element by element, v = the request's
+// state; for every segment in turn its summary is replaced by v and v <- A v + L.  What is left is
+// the request's state after the step, which is stored (the walks for the outputs read the starts only).
+__global__ __launch_bounds__(256) void matrix_memory_prefix_kernel(float* __restrict__ state, long state_stride, int max_slots,
+                                                                   const int* __restrict__ q_start, const int* __restrict__ slots,
+                                                                   float* __restrict__ summaries, const float* __restrict__ m_end,
+                                                                   int heads, int d, int dv, int segs) {
   const int r = blockIdx.x, h = blockIdx.y, slice = blockIdx.z, slices = gridDim.z;
   const int slot = slots[r];
   if (slot < 0 || slot >= max_slots) return;
@@ -263,16 +291,20 @@ __global__ __launch_bounds__(256) void matrix_memory_fold_kernel(float* __restri
   float* Sg = state + (long)slot * state_stride + (long)h * d * dv;
   float* nm = state + (long)slot * state_stride + (long)heads * d * dv + ((long)h * slices + slice) * (d + 1);
   const long sum_floats = mm_summary_floats(d);
-  const float* sums = summaries + (((long)r * segs * heads + h) * slices + slice) * sum_floats;
+  float* sums = summaries + (((long)r * segs * heads + h) * slices + slice) * sum_floats;
   const long sum_stride = (long)heads * slices * sum_floats;
   for (int idx = threadIdx.x; idx < d * MM_COLS + d; idx += blockDim.x) {
     const bool is_n = idx >= d * MM_COLS;
     const int row = is_n ? idx - d * MM_COLS : idx / MM_COLS, c = slice * MM_COLS + idx % MM_COLS;
-    if (!is_n && c >= dv) continue;
-    float* where = is_n ? nm + row : Sg + (long)row * dv + c;
-    float v = *where;
-    for (int s = 0; s < n_seg; ++s) v = fmaf(sums[s * sum_stride + sum_floats - 1], v, sums[s * sum_stride + idx]);
-    *where = v;
+    const bool there = is_n || c < dv;
+    float* where = is_n ? nm + row : Sg + (long)row * dv + (there ? c : 0);
+    float v = there ? *where : 0.f;
+    for (int s = 0; s < n_seg; ++s) {
+      const float A = sums[s * sum_stride + sum_floats - 1], L = sums[s * sum_stride + idx];
+      sums[s * sum_stride + idx] = v;
+      v = fmaf(A, v, L);
+    }
+    if (there) *where = v;
   }
   if (threadIdx.x == 0) nm[d] = m_end[r * heads + h];
 }
@@ -327,12 +359,12 @@ extern "C" int pi_matrix_memory_scan(float* out, long out_stride, const float* p
     MM_PICK(MM_SINGLE);
     return pi_check_launch("matrix_memory_scan");
   }
-  hipLaunchKernelGGL(matrix_memory_gates_kernel, dim3(R, heads), block, 0, stream, coef, m_end, proj, proj_stride, i_off, f_off, i_bias,
+  hipLaunchKernelGGL(matrix_memory_gates_kernel, dim3(R, heads), dim3(MM_GATES_BLOCK), 0, stream, coef, m_end, proj, proj_stride, i_off, f_off, i_bias,
                      f_bias, cap, q_start, slots, state, state_stride, max_slots, heads, d, dv);
   MM_PICK(MM_SUMMARY);
-  MM_PICK(MM_OUTPUT);
-  hipLaunchKernelGGL(matrix_memory_fold_kernel, dim3(R, heads, slices), dim3(256), 0, stream, state, state_stride, max_slots, q_start,
+  hipLaunchKernelGGL(matrix_memory_prefix_kernel, dim3(R, heads, slices), dim3(256), 0, stream, state, state_stride, max_slots, q_start,
                      slots, summaries, m_end, heads, d, dv, segs);
+  MM_PICK(MM_OUTPUT);
 #undef MM_PICK
 #undef MM_GO
   return pi_check_launch("matrix_memory_scan");

@@ -182,7 +182,7 @@ def test_matrix_memory_whole_in_portions_and_token_by_token(sizes):
     """The recurrence through the state slots: whole, in portions of every size down to one token, two requests in
     one step, and a slot used again after it was cleared, against the plain recurrence."""
     from photon_infer_amd import ops
-    H, d, dv, T = sizes              # more than 128 tokens of a request in a step: the walk runs in segments side by side
+    H, d, dv, T = sizes              # more than 64 tokens of a request in a step: the walk runs in segments side by side
     cap = 6.0
     QK, V = H * d, H * dv
     N = 2 * QK + 2 * V + 2 * H
@@ -522,3 +522,41 @@ def test_greedy_generation_through_the_engine(name, dtype, model_dirs):
                     lg = P.forward(cfg, W, prompt + want[:i])[-1]
                     assert float(lg[b] - lg[a]) < 0.05 * float(lg.std()), f"token {i}: {a} instead of {b}"
                     break
+
+
+def test_command_line_and_replayed_decode_steps(model_dirs, tmp_path):
+    """The framework's command serves the design as it serves its others (from a folder, and from a bare configuration
+    with random weights); and decode steps replayed as HIP graphs give the tokens of eager steps, with new requests'
+    prompts in between and states in slots that are used again."""
+    import json
+    import subprocess
+    from photon_infer_amd.engine import ContinuousBatchEngine, EngineOptions
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg, W = P.read_model_folder(model_dirs["P"])
+    prompt = random_tokens(9, cfg["vocab"], 81)
+    want = P.greedy_generate(cfg, W, prompt, 5)
+    proc = subprocess.run([os.path.join(root, "bin", "llama_infer"), model_dirs["P"], "--dtype", "fp32", "--prompt-ids",
+                           ",".join(map(str, prompt)), "--max-new-tokens", "5", "--temperature", "0", "--ignore-eos"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "Architecture: Dafidra" in proc.stdout and f"Generated ids: {','.join(map(str, want))}" in proc.stdout
+    (tmp_path / "cfg").mkdir()
+    json.dump(TD.TINY_Q, open(tmp_path / "cfg" / "config.json", "w"))
+    proc = subprocess.run([os.path.join(root, "bin", "llama_infer"), str(tmp_path / "cfg"), "--random-weights", "--seed", "3",
+                           "--prompt-ids", "5,6,7", "--max-new-tokens", "4", "--ignore-eos"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "Layers: 3" in proc.stdout and "Generated ids:" in proc.stdout
+
+    prompts = [random_tokens(n, cfg["vocab"], 90 + n) for n in (3, 40, 17, 9, 26)]
+
+    def run(use_graphs):
+        eng = ContinuousBatchEngine(model_dirs["P"], EngineOptions(dtype="bfloat16", block_size=16, max_batch=3, max_cache_tokens=1024,
+                                                                   chunk_size=8, max_step_tokens=24, max_model_len=256, use_graphs=use_graphs))
+        assert eng.runner.graph_safe
+        out = eng.generate(prompts, max_new_tokens=20, ignore_eos=True)
+        return out, eng.runner.graphs_captured
+
+    graphs, captured = run(True)
+    eager, none = run(False)
+    assert captured > 0 and none == 0
+    assert [list(o) for o in graphs] == [list(o) for o in eager]

@@ -32,7 +32,7 @@ TINY_Q = {"architecture": "Dafidra", "vocab": 520, "width": 128, "norm": {"eps":
 TINY_Q_INIT = dict(std=0.1, block_size=8)
 
 # R: head sizes the matrix-core kernels take, four heads on one kv head, all groups kept, four of eight experts
-_RL = dict(heads=4, kv_heads=1, dim=64, vdim=64, scale=0.09, mask={"size": 100}, q_temp={"coef": 0.5, "every": 50})
+_RL = dict(heads=4, kv_heads=1, dim=64, vdim=64, scale=0.09, mask={"size": 100}, q_temp={"coef": 0.45, "every": 50})
 _RR = dict(heads=4, dim=32, vdim=32, gate_cap=10.0)
 TINY_R = {"architecture": "Dafidra", "vocab": 776, "width": 256, "norm": {"eps": 1e-5}, "residual_mult": 0.25,
           "layers": [_layer(_RL, _RR, _moe(128, 8, 4, 4, 4)), _layer(_RL, _RR, {"kind": "dense", "ff": 512})]}
