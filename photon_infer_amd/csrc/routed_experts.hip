@@ -290,17 +290,18 @@ extern "C" int pi_grouped_gemm_general(void* C, int c_dtype, long ldc, const voi
 __global__ void combine_choices_kernel(float* __restrict__ out, const float* __restrict__ y, const float* __restrict__ weights,
                                        const int* __restrict__ entry_row, int top, int D, int accumulate) {
   const long t = blockIdx.x;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float acc = 0.f;
-    for (int j = 0; j < top; ++j) acc = fmaf(weights[t * top + j], y[(long)entry_row[t * top + j] * D + d], acc);
-    out[t * D + d] = accumulate ? out[t * D + d] + acc : acc;
-  }
+  const int d = blockIdx.y * blockDim.x + threadIdx.x;
+  if (d >= D) return;
+  float acc = 0.f;
+  for (int j = 0; j < top; ++j) acc = fmaf(weights[t * top + j], y[(long)entry_row[t * top + j] * D + d], acc);
+  out[t * D + d] = accumulate ? out[t * D + d] + acc : acc;
 }
 
 extern "C" int pi_combine_choices(float* out, const float* y, const float* weights, const int* entry_row, int T, int top, int D,
                                   int accumulate, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && top > 0 && D > 0, "combine: bad sizes");
   if (T == 0) return 0;
-  hipLaunchKernelGGL(combine_choices_kernel, dim3(T), dim3(256), 0, stream, out, y, weights, entry_row, top, D, accumulate);
+  PI_REQUIRE((D + 255) / 256 <= 65535, "combine: rows of %d are too long", D);
+  hipLaunchKernelGGL(combine_choices_kernel, dim3(T, (D + 255) / 256), dim3(256), 0, stream, out, y, weights, entry_row, top, D, accumulate);
   return pi_check_launch("combine_choices");
 }

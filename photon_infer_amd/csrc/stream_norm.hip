@@ -50,6 +50,91 @@ __global__ __launch_bounds__(256) void branch_norm_add_kernel(float* __restrict_
   }
 }
 
+// Block-wide sums of two values at once (one trip through LDS for both); `scratch` holds 32 floats.
+__device__ inline void block_sum2(float& a, float& b, float* scratch) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE;
+  const int nwaves = (blockDim.x + PI_WAVE - 1) / PI_WAVE;
+  __syncthreads();
+  if (lane == 0) {
+    scratch[wave] = a;
+    scratch[16 + wave] = b;
+  }
+  __syncthreads();
+  float ta = 0.f, tb = 0.f;
+  for (int w = 0; w < nwaves; ++w) {
+    ta += scratch[w];
+    tb += scratch[16 + w];
+  }
+  a = ta;
+  b = tb;
+}
+
+// The same for rows of whole 16-byte groups, at most VPT groups per thread: a thread keeps its
+// values in registers between the passes, both branches' sums of squares share one reduction,
+// and every access is 16 bytes wide.  Few rows (decode steps) are a matter of latency: as many
+// threads per row as the row has groups.
+template <typename TH, int VPT>
+__global__ __launch_bounds__(1024) void branch_norm_add_wide_kernel(float* __restrict__ x, TH* __restrict__ h, const float* __restrict__ a,
+                                                                    const float* __restrict__ wa, const float* __restrict__ b,
+                                                                    const float* __restrict__ wb, const float* __restrict__ wo,
+                                                                    float eps, float mult, int D) {
+  __shared__ float scratch[32];
+  const long row = blockIdx.x;
+  const int groups = D / 4;
+  float4 va[VPT], vb[VPT], xo[VPT];
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int g = threadIdx.x + v * blockDim.x;
+    const bool in = g < groups;
+    va[v] = in ? reinterpret_cast<const float4*>(a + row * D)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+    vb[v] = (in && b) ? reinterpret_cast<const float4*>(b + row * D)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+    xo[v] = in ? reinterpret_cast<const float4*>(x + row * D)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+    sa = fmaf(va[v].x, va[v].x, sa); sa = fmaf(va[v].y, va[v].y, sa); sa = fmaf(va[v].z, va[v].z, sa); sa = fmaf(va[v].w, va[v].w, sa);
+    sb = fmaf(vb[v].x, vb[v].x, sb); sb = fmaf(vb[v].y, vb[v].y, sb); sb = fmaf(vb[v].z, vb[v].z, sb); sb = fmaf(vb[v].w, vb[v].w, sb);
+  }
+  float sy = sa, unused = 0.f;
+  if (wa) {
+    block_sum2(sa, sb, scratch);
+    const float ra = 1.0f / sqrtf(sa / D + eps);
+    const float rb = b ? 1.0f / sqrtf(sb / D + eps) : 0.f;
+    sy = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+      const int g = threadIdx.x + v * blockDim.x;
+      if (g >= groups) continue;
+      const float4 w1 = reinterpret_cast<const float4*>(wa)[g];
+      float y[4] = {va[v].x * ra * w1.x, va[v].y * ra * w1.y, va[v].z * ra * w1.z, va[v].w * ra * w1.w};
+      if (b) {
+        const float4 w2 = reinterpret_cast<const float4*>(wb)[g];
+        y[0] = 0.5f * (y[0] + vb[v].x * rb * w2.x);
+        y[1] = 0.5f * (y[1] + vb[v].y * rb * w2.y);
+        y[2] = 0.5f * (y[2] + vb[v].z * rb * w2.z);
+        y[3] = 0.5f * (y[3] + vb[v].w * rb * w2.w);
+      }
+      va[v] = make_float4(y[0], y[1], y[2], y[3]);
+      sy = fmaf(y[0], y[0], sy); sy = fmaf(y[1], y[1], sy); sy = fmaf(y[2], y[2], sy); sy = fmaf(y[3], y[3], sy);
+    }
+  }
+  block_sum2(sy, unused, scratch);
+  const float ry = 1.0f / sqrtf(sy / D + eps);
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int g = threadIdx.x + v * blockDim.x;
+    if (g >= groups) continue;
+    const float4 w3 = reinterpret_cast<const float4*>(wo)[g];
+    const float4 r = make_float4(xo[v].x + mult * (va[v].x * ry * w3.x), xo[v].y + mult * (va[v].y * ry * w3.y),
+                                 xo[v].z + mult * (va[v].z * ry * w3.z), xo[v].w + mult * (va[v].w * ry * w3.w));
+    reinterpret_cast<float4*>(x + row * D)[g] = r;
+    if (h) {
+      TH* hp = h + row * D + 4 * (long)g;
+      hp[0] = from_float<TH>(r.x); hp[1] = from_float<TH>(r.y); hp[2] = from_float<TH>(r.z); hp[3] = from_float<TH>(r.w);
+    }
+  }
+}
+
 // x (float32 stream) += mult * norm(...); h (optional, h_dtype) = the new stream.
 // wa == null: a is taken as it is (one branch, no inner norm); b == null: one branch.
 extern "C" int pi_branch_norm_add(float* x, void* h, int h_dtype, const float* a, const float* wa, const float* b,
@@ -58,6 +143,28 @@ extern "C" int pi_branch_norm_add(float* x, void* h, int h_dtype, const float* a
   PI_REQUIRE(x && a && wo, "branch norm: the stream, a branch and the outer weight are needed");
   PI_REQUIRE(!b || (wa && wb), "branch norm: two branches need both their weights");
   if (T == 0) return 0;
+  PI_REQUIRE(!h || h_dtype == PI_BF16 || h_dtype == PI_F32, "branch norm: unsupported activation dtype %d", h_dtype);
+  const bool aligned = D % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)a % 16 == 0 && (!b || (uintptr_t)b % 16 == 0) &&
+                       (uintptr_t)wo % 16 == 0 && (!wa || (uintptr_t)wa % 16 == 0) && (!wb || (uintptr_t)wb % 16 == 0);
+  if (aligned && D / 4 <= 4 * 1024) {
+    const int groups = D / 4;
+    // few rows: a thread per group (latency); many rows: fewer, fatter threads
+    int threads = T <= 512 ? groups : (groups + 3) / 4;
+    threads = threads > 1024 ? 1024 : ((threads + PI_WAVE - 1) / PI_WAVE) * PI_WAVE;
+    const int vpt = (groups + threads - 1) / threads;
+#define BN_GO(TH, V) hipLaunchKernelGGL((branch_norm_add_wide_kernel<TH, V>), dim3(T), dim3(threads), 0, stream, x, (TH*)h, a, wa, b, wb, wo, eps, mult, D)
+#define BN_PICK(TH)            \
+  do {                         \
+    if (vpt <= 1) BN_GO(TH, 1); \
+    else if (vpt <= 2) BN_GO(TH, 2); \
+    else BN_GO(TH, 4);         \
+  } while (0)
+    if (h && h_dtype == PI_BF16) BN_PICK(bf16_t);
+    else BN_PICK(float);
+#undef BN_PICK
+#undef BN_GO
+    return pi_check_launch("branch_norm_add_wide");
+  }
   const size_t lds = (size_t)D * sizeof(float);
   if (h && h_dtype == PI_BF16)
     hipLaunchKernelGGL(branch_norm_add_kernel<bf16_t>, dim3(T), dim3(256), lds, stream, x, (bf16_t*)h, a, wa, b, wb, wo, eps, mult, D);
@@ -91,12 +198,12 @@ extern "C" int pi_cast_stream(void* out, int out_dtype, const float* x, long n, 
 //   gate <- 1 / (1 + exp(-gate))                              -> float32 [T, ng]
 // wq / wk null: no norm of that projection.
 template <typename T>
-__global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
+__global__ __launch_bounds__(1024) void qk_norm_kv_write_kernel(
     T* __restrict__ q_out, long q_stride, float* __restrict__ gate_out, const float* __restrict__ proj, long proj_stride,
     const float* __restrict__ wq, const float* __restrict__ wk, const int* __restrict__ positions, const int* __restrict__ req_of_token,
     float eps, float temp_coef, int temp_every, int nh, int nkv, int hd, int vd, int ng, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages) {
-  __shared__ float scratch[16];
+  __shared__ float scratch[32];
   const long t = blockIdx.x;
   const float* row = proj + t * proj_stride;
   const int QN = nh * hd, KN = nkv * hd, VN = nkv * vd;
@@ -104,8 +211,9 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
   float sq = 0.f, sk = 0.f;
   for (int i = threadIdx.x; i < QN; i += blockDim.x) sq = fmaf(row[i], row[i], sq);
   for (int i = threadIdx.x; i < KN; i += blockDim.x) sk = fmaf(row[QN + i], row[QN + i], sk);
-  const float rq = wq ? 1.0f / sqrtf(block_sum(sq, scratch) / QN + eps) : 1.0f;
-  const float rk = wk ? 1.0f / sqrtf(block_sum(sk, scratch) / KN + eps) : 1.0f;
+  block_sum2(sq, sk, scratch);                   // both sums of squares in one trip through LDS
+  const float rq = wq ? 1.0f / sqrtf(sq / QN + eps) : 1.0f;
+  const float rk = wk ? 1.0f / sqrtf(sk / KN + eps) : 1.0f;
   const float temp = temp_coef != 0.f ? 1.0f + temp_coef * logf((float)((p + 1) / temp_every) + 1.0f) : 1.0f;
   T* qr = q_out + t * q_stride;
   for (int i = threadIdx.x; i < QN; i += blockDim.x) {
@@ -142,7 +250,8 @@ extern "C" int pi_qk_norm_kv_write(void* q_out, long q_stride, float* gate_out, 
              "qk norm: bad cache geometry");
   PI_REQUIRE(ng == 0 || gate_out, "qk norm: gates without a place for them");
   if (T == 0) return 0;
-#define QKN_GO(TT) hipLaunchKernelGGL(qk_norm_kv_write_kernel<TT>, dim3(T), dim3(256), 0, stream, (TT*)q_out, q_stride, gate_out, proj, \
+  const int threads = T <= 64 ? 1024 : 256;      // few tokens (decode steps): the row's passes are a matter of latency
+#define QKN_GO(TT) hipLaunchKernelGGL(qk_norm_kv_write_kernel<TT>, dim3(T), dim3(threads), 0, stream, (TT*)q_out, q_stride, gate_out, proj, \
                                       proj_stride, wq, wk, positions, req_of_token, eps, temp_coef, temp_every, nh, nkv, hd, vd, ng,  \
                                       (TT*)k_cache, (TT*)v_cache, block_table, table_width, page_size, num_pages)
   if (dtype == PI_F32) QKN_GO(float);

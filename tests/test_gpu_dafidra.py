@@ -287,7 +287,8 @@ def model_dirs(tmp_path_factory):
 
 
 _plain = {}
-CLOSE_CALL = 0.08            # router logits: a choice that differs from the plain one must be this close to a tie
+CLOSE_CALL = 0.25            # router logits (their spread is about 1): a bfloat16 choice that differs from the plain one must be
+                             # this close to a tie; float32 runs are held to the plain choices themselves
 
 
 class RouteRecorder:
@@ -388,7 +389,7 @@ def run_checked(runner, steps, out_dir, model_dir, reqs, dtype, what):
     check(got, model_dir, reqs, dtype, what, rec.by_request(steps, P.read_model_folder(model_dir)[0]))
 
 
-LENGTHS = {"P": [1, 26, 90], "Q": [2, 45, 100], "R": [3, 130, 210]}
+LENGTHS = {"P": [1, 26, 90], "Q": [2, 45, 100], "R": [3, 130, 210], "S": [2, 30, 75]}
 
 
 def requests_for(name, seed=0, model_dir=None):
@@ -424,7 +425,7 @@ def test_whole_prompts_and_every_layers_stream(name, dtype, model_dirs, tmp_path
         runner.admit("s")
         runner.step([StepEntry("s", toks, [])])
         for i, (g, w) in enumerate(zip(got, want)):
-            close(g, w, "float32", f"stream after layer {i}", f32=3e-5)
+            close(g, w, "float32", f"stream after layer {i}", f32=1e-4)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

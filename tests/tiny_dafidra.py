@@ -38,7 +38,16 @@ TINY_R = {"architecture": "Dafidra", "vocab": 776, "width": 256, "norm": {"eps":
           "layers": [_layer(_RL, _RR, _moe(128, 8, 4, 4, 4)), _layer(_RL, _RR, {"kind": "dense", "ff": 512})]}
 TINY_R_INIT = dict(std=0.08, block_size=16)
 
-ALL = {"P": (TINY_P, TINY_P_INIT), "Q": (TINY_Q, TINY_Q_INIT), "R": (TINY_R, TINY_R_INIT)}
+# S: sizes that fit no fast kernel: a width that is no multiple of 8, an odd vocabulary, head sizes that are no multiples
+# of 16, three kv heads, three memory heads whose values fill two column groups unevenly, nine experts in three groups of
+# which one is kept, a window shorter than a page, a temperature that changes with every position, no dense layer
+_SL = dict(heads=6, kv_heads=3, dim=24, vdim=40, scale=0.25, mask={"size": 13}, q_temp={"coef": 0.2, "every": 1})
+_SR = dict(heads=3, dim=20, vdim=28, gate_cap=5.0)
+TINY_S = {"architecture": "Dafidra", "vocab": 257, "width": 100, "norm": {"eps": 2e-6}, "residual_mult": 0.4,
+          "layers": [_layer(_SL, _SR, _moe(36, 9, 2, 3, 1)), _layer(_SL, _SR, None), _layer(_SL, _SR, _moe(20, 9, 3, 3, 1))]}
+TINY_S_INIT = dict(std=0.12, block_size=16)
+
+ALL = {"P": (TINY_P, TINY_P_INIT), "Q": (TINY_Q, TINY_Q_INIT), "R": (TINY_R, TINY_R_INIT), "S": (TINY_S, TINY_S_INIT)}
 
 
 def make_model_dir(tmp_path, name: str, seed: int = 0) -> str:
