@@ -196,17 +196,26 @@ extern "C" int pi_cast_stream(void* out, int out_dtype, const float* x, long n, 
 //   k <- k / sqrt(mean over all nkv*hd entries + eps) * wk   -> key pages [page, kv head, slot, hd]
 //   v                                                         -> value pages [page, kv head, vd, slot]
 //   gate <- 1 / (1 + exp(-gate))                              -> float32 [T, ng]
-// wq / wk null: no norm of that projection.
+// wq / wk null: no norm of that projection.  `part` (with `splits` planes of `part_stride` floats, rows of
+// proj_stride columns): the projection as the float32 pieces of a product split over k, instead of `proj`.
 template <typename T>
 __global__ __launch_bounds__(1024) void qk_norm_kv_write_kernel(
     T* __restrict__ q_out, long q_stride, float* __restrict__ gate_out, const float* __restrict__ proj, long proj_stride,
     const float* __restrict__ wq, const float* __restrict__ wk, const int* __restrict__ positions, const int* __restrict__ req_of_token,
     float eps, float temp_coef, int temp_every, int nh, int nkv, int hd, int vd, int ng, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages) {
+    T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages,
+    const float* __restrict__ part, int splits, long part_stride) {
   __shared__ float scratch[32];
+  extern __shared__ float staged[];              // the token's row, when it comes in pieces
   const long t = blockIdx.x;
   const float* row = proj + t * proj_stride;
   const int QN = nh * hd, KN = nkv * hd, VN = nkv * vd;
+  if (part) {
+    // the projection is still split over k: its float32 pieces are added here, in split order, once per element
+    for (int i = threadIdx.x; i < QN + KN + VN + ng; i += blockDim.x) staged[i] = split_sum(part, splits, part_stride, t * proj_stride + i);
+    __syncthreads();
+    row = staged;
+  }
   const int p = positions[t];
   float sq = 0.f, sk = 0.f;
   for (int i = threadIdx.x; i < QN; i += blockDim.x) sq = fmaf(row[i], row[i], sq);
@@ -242,18 +251,23 @@ extern "C" int pi_qk_norm_kv_write(void* q_out, long q_stride, float* gate_out, 
                                    const float* wq, const float* wk, const int* positions, const int* req_of_token, float eps,
                                    float temp_coef, int temp_every, int T, int nh, int nkv, int hd, int vd, int ng,
                                    void* k_cache, void* v_cache, const int* block_table, int table_width, int page_size,
-                                   long num_pages, hipStream_t stream) {
+                                   long num_pages, const float* part, int splits, long part_stride, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && ng >= 0, "qk norm: bad sizes");
   PI_REQUIRE(proj_stride >= (long)nh * hd + (long)nkv * (hd + vd) + ng, "qk norm: projection rows of %ld hold no q, k, v and gates", proj_stride);
   PI_REQUIRE(temp_coef == 0.f || temp_every > 0, "qk norm: the temperature's period must be positive, got %d", temp_every);
   PI_REQUIRE(!k_cache || (v_cache && block_table && req_of_token && table_width > 0 && page_size > 0 && num_pages > 0),
              "qk norm: bad cache geometry");
   PI_REQUIRE(ng == 0 || gate_out, "qk norm: gates without a place for them");
+  PI_REQUIRE((proj != nullptr) != (part != nullptr), "qk norm: give the projection as a tensor or as pieces");
+  PI_REQUIRE(!part || (splits >= 1 && part_stride >= (long)T * proj_stride), "qk norm: bad pieces (%d planes of %ld floats)", splits, part_stride);
+  const long row_floats = (long)nh * hd + (long)nkv * (hd + vd) + ng;
+  PI_REQUIRE(!part || row_floats * 4 <= 60000, "qk norm: rows of %ld floats in pieces do not fit the staging memory", row_floats);
+  const size_t lds = part ? (size_t)row_floats * sizeof(float) : 0;
   if (T == 0) return 0;
   const int threads = T <= 64 ? 1024 : 256;      // few tokens (decode steps): the row's passes are a matter of latency
-#define QKN_GO(TT) hipLaunchKernelGGL(qk_norm_kv_write_kernel<TT>, dim3(T), dim3(threads), 0, stream, (TT*)q_out, q_stride, gate_out, proj, \
+#define QKN_GO(TT) hipLaunchKernelGGL(qk_norm_kv_write_kernel<TT>, dim3(T), dim3(threads), lds, stream, (TT*)q_out, q_stride, gate_out, proj, \
                                       proj_stride, wq, wk, positions, req_of_token, eps, temp_coef, temp_every, nh, nkv, hd, vd, ng,  \
-                                      (TT*)k_cache, (TT*)v_cache, block_table, table_width, page_size, num_pages)
+                                      (TT*)k_cache, (TT*)v_cache, block_table, table_width, page_size, num_pages, part, splits, part_stride)
   if (dtype == PI_F32) QKN_GO(float);
   else if (dtype == PI_BF16) QKN_GO(bf16_t);
   else return pi_fail("qk norm: unsupported dtype %d", dtype);

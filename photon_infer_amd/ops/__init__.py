@@ -539,14 +539,19 @@ def qk_norm_kv_write(q_out: torch.Tensor, gate_out: Optional[torch.Tensor], proj
                      w_k: Optional[torch.Tensor], ctx, eps: float, temp_coef: float, temp_every: int, num_heads: int,
                      num_kv_heads: int, head_dim: int, value_dim: int, num_gates: int, k_cache: Optional[torch.Tensor],
                      v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor], page_size: int) -> None:
-    """From float32 projection rows [q | k | v | gates]: queries and keys each normalised over their
+    """From float32 projection rows [q | k | v | gates] (a tensor, or ``Partials``: the product still split over k,
+    whose pieces are added here): queries and keys each normalised over their
     WHOLE row (all heads at once; weights float32, None: no norm), queries times the position's
     temperature 1 + coef * ln(floor((p + 1) / every) + 1), keys and values into their pages,
     gates through a sigmoid into ``gate_out`` (float32 [T, num_gates])."""
-    _gpu(q_out, gate_out, proj, w_q, w_k, k_cache, v_cache, block_table)
+    pieces = proj if isinstance(proj, Partials) else None
+    _gpu(q_out, gate_out, pieces.part if pieces is not None else proj, w_q, w_k, k_cache, v_cache, block_table)
     T = q_out.shape[0]
     QN, KN, VN = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * value_dim
-    if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < QN + KN + VN + num_gates:
+    if pieces is not None:
+        if pieces.M != T or pieces.N < QN + KN + VN + num_gates:
+            raise KernelError(f"qk norm: pieces [{pieces.M}, {pieces.N}] do not hold q, k, v and gates of {T} tokens")
+    elif proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < QN + KN + VN + num_gates:
         raise KernelError(f"qk norm: projection must be float32 [{T}, >= {QN + KN + VN + num_gates}], got {proj.dtype} {tuple(proj.shape)}")
     if q_out.shape[1] != QN:
         raise KernelError(f"qk norm: q has {q_out.shape[1]} columns, expected {QN}")
@@ -561,10 +566,13 @@ def qk_norm_kv_write(q_out: torch.Tensor, gate_out: Optional[torch.Tensor], proj
             raise KernelError("qk norm: block table must be contiguous int32 [requests, width]")
     _i32(ctx.positions, "positions", T)
     _i32(ctx.req_of_token, "req_of_token", T)
-    _lib.call("core", "pi_qk_norm_kv_write", q_out.data_ptr(), _rows(q_out, "q"), _ptr(gate_out), _dt(q_out), proj.data_ptr(),
-              _rows(proj, "projection"), _ptr(w_q), _ptr(w_k), ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), float(eps),
+    _lib.call("core", "pi_qk_norm_kv_write", q_out.data_ptr(), _rows(q_out, "q"), _ptr(gate_out), _dt(q_out),
+              None if pieces is not None else proj.data_ptr(), pieces.N if pieces is not None else _rows(proj, "projection"),
+              _ptr(w_q), _ptr(w_k), ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), float(eps),
               float(temp_coef), int(temp_every), T, num_heads, num_kv_heads, head_dim, value_dim, num_gates, _ptr(k_cache),
-              _ptr(v_cache), _ptr(block_table), block_table.shape[1] if k_cache is not None else 0, page_size, pages, _stream())
+              _ptr(v_cache), _ptr(block_table), block_table.shape[1] if k_cache is not None else 0, page_size, pages,
+              pieces.part.data_ptr() if pieces is not None else None, pieces.splits if pieces is not None else 0,
+              pieces.M * pieces.N if pieces is not None else 0, _stream())
 
 
 # ----------------------------------------------------------------------------- matrix memory

@@ -23,7 +23,7 @@ _SIGNATURES = {
         "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, P],
         "pi_branch_norm_add": [P, P, I, P, P, P, P, P, F, F, I, I, P],
         "pi_cast_stream": [P, I, P, L, P],
-        "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P],
+        "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, L, P],
         "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, I, I, P, L, P],
         "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, P],
         "pi_route": [P, P, P, L, I, I, I, I, I, I, P],

@@ -85,8 +85,8 @@ class SinkWindowAttention(Mixer):
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         T, ws = h.shape[0], ctx.workspace
         table = ctx.block_tables[cache.group]
-        proj = torch.empty((T, self.w_in.shape[0]), dtype=torch.float32, device=h.device)
-        ops.gemm(proj, h, self.w_in, ws=ws)
+        # a float32 tensor, or - where the product was split over k - its pieces, which the next kernel adds
+        proj = ops.qkv_projection(h, self.w_in, torch.float32, ws)
         q = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
         gate = torch.empty((T, self.num_heads), dtype=torch.float32, device=h.device) if self.output_gate else None
         ops.qk_norm_kv_write(q, gate, proj, self.w_qn, self.w_kn, ctx, self.eps, self.temp_coef, self.temp_every,

@@ -98,6 +98,34 @@ def test_attention_mechanisms_alone(dtype, sizes):
     close(out, ref, dtype, "attention output", bf16=3e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_qk_norm_adds_the_pieces_of_a_split_projection(dtype):
+    """The projection as the float32 pieces of a product split over k gives what their sum gives as a tensor:
+    queries, gates and the pages' keys and values, bit for bit."""
+    from photon_infer_amd import ops
+    from photon_infer_amd.ops import Partials
+    H, G, d, dv, page, T, splits = 4, 2, 24, 40, 8, 11, 5
+    N = H * d + G * d + G * dv + H
+    td = TORCH[dtype]
+    part = randn(splits, T, N, seed=1).float().to(DEV).contiguous()
+    whole = torch.zeros((T, N), dtype=torch.float32, device=DEV)
+    for s_ in range(splits):         # in split order, as the kernel adds them
+        whole += part[s_]
+    ctx = attention_ctx([T], [T + 20], td)
+    table = torch.arange(8, dtype=torch.int32, device=DEV).flip(0).view(1, 8).contiguous()
+    wq, wk = (randn(H * d, seed=2) + 2.0).float().to(DEV), (randn(G * d, seed=3) + 2.0).float().to(DEV)
+    got = []
+    for proj in (whole, Partials(part.view(-1), splits, T, N)):
+        q = torch.zeros((T, H * d), dtype=td, device=DEV)
+        gate = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+        kc = torch.zeros((8, G, page, d), dtype=td, device=DEV)
+        vc = torch.zeros((8, G, dv, page), dtype=td, device=DEV)
+        ops.qk_norm_kv_write(q, gate, proj, wq, wk, ctx, 1e-5, 0.3, 4, H, G, d, dv, H, kc, vc, table, page)
+        got.append((q, gate, kc, vc))
+    for a, b in zip(*got):
+        assert torch.equal(a, b) and float(a.float().abs().max()) > 0
+
+
 @pytest.mark.parametrize("window", [0, 100, 700])
 @pytest.mark.parametrize("hd,H,G", [(64, 8, 2), (128, 4, 4), (32, 2, 1)])
 def test_matrix_core_attention_with_options_against_the_general_kernel(hd, H, G, window):
@@ -561,3 +589,38 @@ def test_command_line_and_replayed_decode_steps(model_dirs, tmp_path):
     eager, none = run(False)
     assert captured > 0 and none == 0
     assert [list(o) for o in graphs] == [list(o) for o in eager]
+
+
+def test_kernels_chosen_at_real_widths_against_the_general_kernels(tmp_path):
+    """A model wide enough that the bfloat16 engine takes what it takes at real sizes - products split over k whose pieces
+    the q/k norm kernel adds, tile products for the prompt, the memory walked in segments, the matrix-core attention -
+    against the same engine on the general kernels: a 300-token prompt, a mixed step and decode steps of a batch."""
+    from photon_infer_amd import ops
+    from photon_infer_amd.config import DafidraConfig
+    from photon_infer_amd.engine.replay import make_runner
+    from photon_infer_amd.engine.step import StepEntry
+    from photon_infer_amd.weights import write_random_model
+    left = dict(heads=16, kv_heads=4, dim=64, vdim=64, scale=0.1, mask={"size": 200}, q_temp={"coef": 0.3, "every": 64})
+    right = dict(heads=4, dim=64, vdim=128, gate_cap=9.0)
+    layer = {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": {"kind": "dense", "ff": 2048}}
+    raw = {"architecture": "Dafidra", "vocab": 1000, "width": 1024, "norm": {"eps": 1e-5}, "residual_mult": 0.6, "layers": [layer, layer]}
+    d = write_random_model(DafidraConfig.from_dict(raw), str(tmp_path / "wide"), seed=2, std=0.03, norm_init="uniform", dtype="bfloat16")
+    prompts = {"a": random_tokens(300, 1000, 1), "b": random_tokens(70, 1000, 2), "c": random_tokens(5, 1000, 3)}
+    outs = []
+    for fast in (True, False):
+        prev = ops.use_fast_kernels(fast)
+        try:
+            r = make_runner(d, "bfloat16", 1024, 16)
+            for rid in prompts:
+                r.admit(rid)
+            got = [r.step([StepEntry("a", prompts["a"], [0, 150, 299])]),
+                   r.step([StepEntry("b", prompts["b"][:60], [59]), StepEntry("c", prompts["c"], [4]), StepEntry("a", [7], [0])])]
+            for k in range(3):
+                got.append(r.step([StepEntry("a", [8 + k], [0]), StepEntry("b", [prompts["b"][60 + k]], [0]), StepEntry("c", [9 + k], [0])]))
+            outs.append(torch.cat(got).float().cpu())
+            if fast:
+                assert r.workspace.counts["qkv_pieces"] > 0, dict(r.workspace.counts)
+        finally:
+            ops.use_fast_kernels(prev)
+    err = float((outs[0] - outs[1]).abs().max())
+    assert err <= 0.04 * float(outs[1].std()) + 0.02, (err, float(outs[1].std()))
