@@ -425,10 +425,6 @@ def requests_for(name, seed=0, model_dir=None):
     return {f"r{i}": random_tokens(n, vocab, seed * 100 + i) for i, n in enumerate(LENGTHS[name])}
 
 
-def clear_tokens(model_dir, n, vocab, seed):
-    return random_tokens(n, vocab, seed)
-
-
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", list(TD.ALL))
 def test_whole_prompts_and_every_layers_stream(name, dtype, model_dirs, tmp_path):
@@ -487,7 +483,7 @@ def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, model_dirs, 
     out a step; a finished request's pages and slot go to the next one.  Each must come out as it does alone."""
     vocab = TD.ALL[name][0]["vocab"]
     lengths = [70, 33, 5, 120, 64, 18, 91]
-    reqs = {f"m{i}": clear_tokens(model_dirs[name], n, vocab, 50 + i) for i, n in enumerate(lengths)}
+    reqs = {f"m{i}": random_tokens(n, vocab, 50 + i) for i, n in enumerate(lengths)}
     rng = np.random.default_rng(7)
     waiting, live, at, steps = list(reqs), [], {}, []
     while waiting or live:
@@ -518,7 +514,7 @@ def test_long_decoding_gives_pages_back_and_keeps_its_state(name, model_dirs, tm
     """400 tokens one by one: many windows pass, the windowed cache group hands pages back while the request runs, and
     the memory's state is all that remembers the early tokens."""
     vocab = TD.ALL[name][0]["vocab"]
-    toks = clear_tokens(model_dirs[name], 400, vocab, 9)
+    toks = random_tokens(400, vocab, 9)
     steps = cut_steps("long", toks, [3] + [1] * 397)
     runner = runner_for(model_dirs[name], name, "float32", 128)      # far fewer pages than 400 tokens: only a window's worth is live
     check(run_trace(runner, steps, str(tmp_path)), model_dirs[name], {"long": toks}, "float32", "long decoding")
