@@ -1,5 +1,6 @@
 from .base import ConfigReader, architecture_name, read_config_json
 from .dafidra import DafidraConfig
 from .llama import LlamaConfig, RopeScaling
+from .rorevik import RorevikConfig
 
-__all__ = ["ConfigReader", "architecture_name", "read_config_json", "LlamaConfig", "RopeScaling", "DafidraConfig"]
+__all__ = ["ConfigReader", "architecture_name", "read_config_json", "LlamaConfig", "RopeScaling", "DafidraConfig", "RorevikConfig"]

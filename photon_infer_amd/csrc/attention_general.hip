@@ -14,7 +14,9 @@
 //   * a distance bias: slope[head] * (p - t) is taken off the scaled score of key t;
 //   * a sink per head: exp(sink[head]) joins the denominator once; it has no key and no value,
 //     is not scaled and gets no bias;
-//   * an output gate: head h's output at token t is multiplied by gate[t, h] (float32).
+//   * an output gate: head h's output at token t is multiplied by gate[t, h] (float32);
+//   * a cap on the scores: the scaled score s becomes softcap * tanh(s / softcap) (0: none), before any bias;
+//   * a factor on every output (out_mult; 1: none), applied in float32 before the one rounding.
 //
 // Keys are visited 64 at a time with the usual running maximum / running sum, so the
 // result for a token depends only on that token's position and its request's pages.
@@ -33,7 +35,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     const T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ req_of_token, const int* __restrict__ positions, int nh, int nkv, int hd, int page_size,
     float scale, int window, long num_pages, float* __restrict__ part, int vd, const float* __restrict__ slopes,
-    const float* __restrict__ sinks, const float* __restrict__ gate) {
+    const float* __restrict__ sinks, const float* __restrict__ gate, float softcap, float out_mult) {
   __shared__ float qs[PI_MAX_HEAD_DIM];
   __shared__ float ps[PI_WAVE];
   __shared__ long voff[PI_WAVE];   // values are stored [page, kv_head, head_dim, slot]
@@ -82,6 +84,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
           for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
         }
         s = dot * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         if (slopes) s -= slope * (float)(p - key);
       } else {
         s = __builtin_nanf("");  // a key without a page: make it visible, never read outside the pool
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) acc[i] *= corr;
   }
   T* o = out + t * out_stride + (long)h * vd;
-  const float inv = (gate ? gate[t * nh + h] : 1.0f) / l;
+  const float inv = out_mult * (gate ? gate[t * nh + h] : 1.0f) / l;
 #pragma unroll
   for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
     const int d = lane + i * PI_WAVE;
@@ -168,7 +171,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
 template <typename T>
 __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ part,
                                                                    int nh, int hd, int splits, const float* __restrict__ sinks,
-                                                                   const float* __restrict__ gate) {
+                                                                   const float* __restrict__ gate, float out_mult) {
   const long t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* base = part + ((long)t * nh + h) * splits * (hd + 2);
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict
     }
   }
   T* o = out + t * out_stride + (long)h * hd;
-  const float inv = (gate ? gate[t * nh + h] : 1.0f) / l;
+  const float inv = out_mult * (gate ? gate[t * nh + h] : 1.0f) / l;
 #pragma unroll
   for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
     const int d = lane + i * PI_WAVE;
@@ -212,7 +215,7 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
                                           const int* req_of_token, const int* positions, int T, int nh, int nkv, int hd,
                                           int page_size, float scale, int window, long num_pages, int splits, void* part,
                                           long part_elems, int vd, const float* slopes, const float* sinks, const float* gate,
-                                          hipStream_t stream) {
+                                          float softcap, float out_mult, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention: heads %d must be a positive multiple of kv heads %d", nh, nkv);
   PI_REQUIRE(hd > 0 && hd <= PI_MAX_HEAD_DIM, "attention: head_dim %d must be at most %d", hd, PI_MAX_HEAD_DIM);
   PI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "attention: bad cache geometry page_size=%d table_width=%d pages=%ld", page_size, table_width, num_pages);
@@ -227,18 +230,18 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
   if (dtype == PI_F32)
     hipLaunchKernelGGL(paged_attention_general_kernel<float>, grid, block, 0, stream, (float*)out, out_stride, (const float*)q,
                        q_stride, (const float*)k_cache, (const float*)v_cache, block_table, table_width, req_of_token,
-                       positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate);
+                       positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(paged_attention_general_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, out_stride,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width,
-                       req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate);
+                       req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult);
   else
     return pi_fail("attention: unsupported dtype %d", dtype);
   if (pi_check_launch("paged_attention_general")) return -1;
   if (splits == 1) return 0;
   if (dtype == PI_F32)
-    hipLaunchKernelGGL(merge_key_ranges_kernel<float>, dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate);
+    hipLaunchKernelGGL(merge_key_ranges_kernel<float>, dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
   else
-    hipLaunchKernelGGL(merge_key_ranges_kernel<bf16_t>, dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate);
+    hipLaunchKernelGGL(merge_key_ranges_kernel<bf16_t>, dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
   return pi_check_launch("merge_key_ranges");
 }

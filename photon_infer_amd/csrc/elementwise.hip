@@ -35,6 +35,41 @@ extern "C" int pi_embedding(float* out, const void* table, int table_dtype, cons
   return pi_check_launch("embedding");
 }
 
+// out[t, :] = float(table[ids[t], :]) * scale + float(pos_table[positions[t], :]): an embedding that is
+// scaled and then meets a learned position vector (not scaled).  A position beyond the table gives a
+// NaN row, like an id beyond the vocabulary.
+template <typename TW>
+__global__ void embedding_positions_kernel(float* __restrict__ out, const TW* __restrict__ table, const int* __restrict__ ids,
+                                           const TW* __restrict__ pos_table, const int* __restrict__ positions, float scale,
+                                           int D, int V, int P) {
+  const long t = blockIdx.x;
+  const int id = ids[t], p = positions[t];
+  float* o = out + t * D;
+  if (id < 0 || id >= V || p < 0 || p >= P) {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = __builtin_nanf("");
+    return;
+  }
+  const TW* row = table + (long)id * D;
+  const TW* prow = pos_table + (long)p * D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = fmaf(to_float(row[i]), scale, to_float(prow[i]));
+}
+
+extern "C" int pi_embedding_positions(float* out, const void* table, const void* pos_table, int table_dtype, const int* ids,
+                                      const int* positions, float scale, int T, int D, int V, int P, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && D > 0 && V > 0 && P > 0, "embedding: bad sizes T=%d D=%d V=%d positions=%d", T, D, V, P);
+  if (T == 0) return 0;
+  const int threads = D >= 256 ? 256 : 64;
+  if (table_dtype == PI_F32)
+    hipLaunchKernelGGL(embedding_positions_kernel<float>, dim3(T), dim3(threads), 0, stream, out, (const float*)table, ids,
+                       (const float*)pos_table, positions, scale, D, V, P);
+  else if (table_dtype == PI_BF16)
+    hipLaunchKernelGGL(embedding_positions_kernel<bf16_t>, dim3(T), dim3(threads), 0, stream, out, (const bf16_t*)table, ids,
+                       (const bf16_t*)pos_table, positions, scale, D, V, P);
+  else
+    return pi_fail("embedding: unsupported table dtype %d", table_dtype);
+  return pi_check_launch("embedding_positions");
+}
+
 // ------------------------------------------------------------------ RMS norm
 // y[m, :] = w * (x[r, :] * (1 / sqrt(mean(x[r, :]^2) + eps))), r = rows ? rows[m] : m.
 // Sum of squares, root and scaling in float32; one rounding on store.
@@ -239,6 +274,44 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
   return pi_check_launch("swiglu");
 }
 
+// ------------------------------------------------------------------ clamped gated unit with biases
+// g = min(gate + bg, limit), u = clamp(up + bu, -limit, limit), out = g * sigmoid(alpha * g) * (u + 1).
+// The gate and up products lie in halves of a row ([gate | up]) in TI; biases and arithmetic are
+// float32.  Optionally the stream's row gets a bias added on the way (x[t, :] += xb): the bias of
+// the product that follows, which then only accumulates.
+template <typename TO, typename TI, typename TB>
+__global__ void clamped_glu_kernel(TO* __restrict__ out, const TI* __restrict__ gu, const TB* __restrict__ bg,
+                                   const TB* __restrict__ bu, float limit, float alpha, int I, float* __restrict__ x,
+                                   const TB* __restrict__ xb, int D) {
+  const long t = blockIdx.x;
+  const TI* row = gu + t * 2 * I;
+  for (int i = threadIdx.x; i < I; i += blockDim.x) {
+    const float g = fminf(to_float(row[i]) + to_float(bg[i]), limit);
+    const float u = fminf(fmaxf(to_float(row[I + i]) + to_float(bu[i]), -limit), limit);
+    out[t * I + i] = from_float<TO>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+  }
+  if (x)
+    for (int i = threadIdx.x; i < D; i += blockDim.x) x[t * D + i] += to_float(xb[i]);
+}
+
+extern "C" int pi_clamped_glu(void* out, int out_dtype, const void* gu, int gu_dtype, const void* bg, const void* bu,
+                              const void* xb, int b_dtype, float limit, float alpha, int T, int I, float* x, int D,
+                              hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && I > 0 && (!x || (xb && D > 0)), "clamped unit: bad sizes T=%d I=%d D=%d", T, I, D);
+  if (T == 0) return 0;
+  const dim3 grid(T), block(256);
+#define PI_GLU(TO_, TI_, TB_)                                                                                               \
+  hipLaunchKernelGGL((clamped_glu_kernel<TO_, TI_, TB_>), grid, block, 0, stream, (TO_*)out, (const TI_*)gu, (const TB_*)bg, \
+                     (const TB_*)bu, limit, alpha, I, x, (const TB_*)xb, D)
+  if (out_dtype == PI_F32 && gu_dtype == PI_F32 && b_dtype == PI_F32) PI_GLU(float, float, float);
+  else if (out_dtype == PI_BF16 && gu_dtype == PI_F32 && b_dtype == PI_BF16) PI_GLU(bf16_t, float, bf16_t);
+  else if (out_dtype == PI_BF16 && gu_dtype == PI_BF16 && b_dtype == PI_BF16) PI_GLU(bf16_t, bf16_t, bf16_t);
+  else if (out_dtype == PI_BF16 && gu_dtype == PI_F32 && b_dtype == PI_F32) PI_GLU(bf16_t, float, float);
+  else return pi_fail("clamped unit: unsupported dtypes out=%d in=%d bias=%d", out_dtype, gu_dtype, b_dtype);
+#undef PI_GLU
+  return pi_check_launch("clamped_glu");
+}
+
 // ------------------------------------------------------------------ rotation + cache write
 // One wave per (token, head).  Heads 0..nh-1 are queries (rotated in place); then, when
 // the layer writes its cache, nkv key heads (rotated, stored to the page of the token's
@@ -290,7 +363,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token, const float* __restrict__ table,
     int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages,
-    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col) {
+    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col, int vd) {
   const long t = blockIdx.x;
   const int h = blockIdx.y * 4 + threadIdx.x / PI_WAVE;
   const int lane = threadIdx.x % PI_WAVE;
@@ -299,6 +372,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   long dst_stride = 1;        // element stride of the destination (values are stored transposed)
   const T* src = nullptr;
   int col = 0;
+  int width = hd;             // features of this head (values may be wider or narrower than keys)
   bool rotate = rotary_dim > 0;
   if (h < nh) {
     dst = q + t * q_stride + (long)h * hd;
@@ -315,11 +389,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     const long page = block_table[(long)r * table_width + blk];
     if (page < 0 || page >= num_pages) return;  // the host checks tables; never write outside the pool
     if (is_v) {
-      src = v ? v + t * v_stride + (long)g * hd : nullptr;
-      col = v_col + g * hd;
-      dst = v_cache + (page * nkv + g) * (long)page_size * hd + (pos % page_size);
+      src = v ? v + t * v_stride + (long)g * vd : nullptr;
+      col = v_col + g * vd;
+      dst = v_cache + (page * nkv + g) * (long)page_size * vd + (pos % page_size);
       dst_stride = page_size;
       rotate = false;
+      width = vd;
     } else {
       src = k ? k + t * k_stride + (long)g * hd : nullptr;
       col = k_col + g * hd;
@@ -343,7 +418,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     if (part || dst != src)
       for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
   } else if (part || dst != src) {
-    for (int i = lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
+    for (int i = lane; i < width; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
   }
 }
 
@@ -480,7 +555,9 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                                 int rotary_dim, int interleaved, int T, int nh, int nkv, int hd, int write_kv,
                                 void* k_cache, void* v_cache, const int* block_table, int table_width,
                                 int page_size, long num_pages, const float* part, int splits, int ncols, int q_col,
-                                int k_col, int v_col, hipStream_t stream) {
+                                int k_col, int v_col, int vd, hipStream_t stream) {
+  if (vd <= 0) vd = hd;
+  PI_REQUIRE(vd <= 256, "rope_kv_write: value width %d must be at most 256", vd);
   PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd <= 256, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
   PI_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, hd);
   PI_REQUIRE(rotary_dim == 0 || table != nullptr, "rope_kv_write: rotation asked for without a cos / sin table");
@@ -497,7 +574,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                               : (!write_kv || (k_stride % 8 == 0 && ((uintptr_t)k % 16 == 0)));
   const bool aligned = hd % 16 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && (!table || (uintptr_t)table % 16 == 0) &&
                        source_ok && (!write_kv || (((uintptr_t)k_cache % 16 == 0) && ((uintptr_t)v_cache % 8 == 0) && page_size % 4 == 0));
-  if (dtype == PI_BF16 && usual && aligned && T >= 16) {
+  if (dtype == PI_BF16 && usual && aligned && T >= 16 && vd == hd) {
     const int nkv_w = write_kv ? nkv : 0;
     const long rot_items = (long)T * (nh + nkv_w) * (hd / 16);
     const long v_items = write_kv ? (long)((T + 3) / 4) * nkv * hd : 0;
@@ -517,12 +594,12 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
     hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)q, q_stride, (const float*)k, k_stride,
                        (const float*)v, v_stride, positions, req_of_token, table, rotary_dim, interleaved, nh, nkv_write,
                        nkv, hd, (float*)k_cache, (float*)v_cache, block_table, table_width, page_size, num_pages, part,
-                       splits, part_stride, ncols, q_col, k_col, v_col);
+                       splits, part_stride, ncols, q_col, k_col, v_col, vd);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)q, q_stride, (const bf16_t*)k, k_stride,
                        (const bf16_t*)v, v_stride, positions, req_of_token, table, rotary_dim, interleaved, nh, nkv_write,
                        nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table, table_width, page_size, num_pages, part,
-                       splits, part_stride, ncols, q_col, k_col, v_col);
+                       splits, part_stride, ncols, q_col, k_col, v_col, vd);
   else
     return pi_fail("rope_kv_write: unsupported dtype %d", dtype);
   return pi_check_launch("rope_kv_write");

@@ -98,15 +98,26 @@ def check_general_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: i
 
 
 # ----------------------------------------------------------------------------- ops
-def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
-    """out[t, :] = float32(table[ids[t], :])."""
-    _gpu(out, table, ids)
+def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0,
+              pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
+    """out[t, :] = float32(table[ids[t], :]); with a learned position table,
+    out[t, :] = table[ids[t], :] * scale + pos_table[positions[t], :]."""
+    _gpu(out, table, ids, pos_table, positions)
     T, D = out.shape
     if out.dtype != torch.float32 or not out.is_contiguous():
         raise KernelError("embedding: output must be contiguous float32")
     if table.dim() != 2 or table.shape[1] != D or not table.is_contiguous():
         raise KernelError(f"embedding: table shape {tuple(table.shape)} does not match width {D}")
     _i32(ids, "embedding ids", T)
+    if pos_table is not None:
+        if pos_table.dim() != 2 or pos_table.shape[1] != D or not pos_table.is_contiguous() or pos_table.dtype != table.dtype:
+            raise KernelError(f"embedding: position table {tuple(pos_table.shape)} {pos_table.dtype} does not match [*, {D}] {table.dtype}")
+        _i32(positions, "embedding positions", T)
+        _lib.call("core", "pi_embedding_positions", out.data_ptr(), table.data_ptr(), pos_table.data_ptr(), _dt(table), ids.data_ptr(),
+                  positions.data_ptr(), float(scale), T, D, table.shape[0], pos_table.shape[0], _stream())
+        return
+    if scale != 1.0:
+        raise KernelError("embedding: a scale comes with a position table")
     _lib.call("core", "pi_embedding", out.data_ptr(), table.data_ptr(), _dt(table), ids.data_ptr(), T, D,
               table.shape[0], _stream())
 
@@ -302,8 +313,10 @@ def qkv_projection(h: torch.Tensor, w_qkv: torch.Tensor, dtype: torch.dtype, ws:
 def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], positions: torch.Tensor,
                   req_of_token: torch.Tensor, rotary, num_heads: int, num_kv_heads: int, head_dim: int,
                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                  block_table: Optional[torch.Tensor], page_size: int, pieces=None, write_kv: Optional[bool] = None) -> None:
+                  block_table: Optional[torch.Tensor], page_size: int, pieces=None, write_kv: Optional[bool] = None,
+                  value_dim: Optional[int] = None) -> None:
     """Rotate q in place by each token's position; rotate k and store k, v into the pages.
+    ``value_dim``: the width of a value head when it differs from ``head_dim``.
 
     ``rotary`` = (inv_freq float32 [R/2] or the step's cos / sin table [T, R], R, interleaved), or
     None for no rotation.
@@ -314,7 +327,11 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     """
     _gpu(q, k, v, positions, req_of_token, k_cache, v_cache, block_table)
     T = q.shape[0]
-    check_attention_sizes(num_heads, num_kv_heads, head_dim)
+    vd = head_dim if value_dim is None else int(value_dim)
+    if vd == head_dim:
+        check_attention_sizes(num_heads, num_kv_heads, head_dim)
+    else:
+        check_general_attention_sizes(num_heads, num_kv_heads, head_dim, vd)
     if q.shape[1] != num_heads * head_dim:
         raise KernelError(f"rope: q has {q.shape[1]} columns, expected {num_heads * head_dim}")
     _i32(positions, "positions", T)
@@ -322,15 +339,15 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         write = bool(write_kv)
         table_ptr, rdim, inter, _keep = _rotary_args(rotary, positions, T)
         q_size, kv_size = num_heads * head_dim, num_kv_heads * head_dim
-        if pieces.M != T or pieces.N < q_size + (2 * kv_size if write else 0):
+        if pieces.M != T or pieces.N < q_size + (kv_size + num_kv_heads * vd if write else 0):
             raise KernelError(f"rope: pieces [{pieces.M}, {pieces.N}] do not hold q, k, v of {T} tokens")
-        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype) if write else 0
+        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype, vd) if write else 0
         _lib.call(
             "core", "pi_rope_kv_write", q.data_ptr(), _rows(q, "q"), None, 0, None, 0, _dt(q), positions.data_ptr(),
             _ptr(req_of_token) if write else None, table_ptr, rdim, int(bool(inter)), T, num_heads, num_kv_heads,
             head_dim, int(write), _ptr(k_cache) if write else None, _ptr(v_cache) if write else None,
             _ptr(block_table) if write else None, block_table.shape[1] if write else 0, page_size if write else 0, pages,
-            pieces.part.data_ptr(), pieces.splits, pieces.N, 0, q_size, q_size + kv_size, _stream())
+            pieces.part.data_ptr(), pieces.splits, pieces.N, 0, q_size, q_size + kv_size, vd, _stream())
         return
     write = k is not None
     table_ptr, rdim, inter, _keep = _rotary_args(rotary, positions, T)
@@ -338,9 +355,10 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         return
     pages = 0
     if write:
-        if v is None or k.shape != (T, num_kv_heads * head_dim) or v.shape != k.shape or k.dtype != q.dtype or v.dtype != q.dtype:
-            raise KernelError(f"rope: k/v must be [{T}, {num_kv_heads * head_dim}] of {q.dtype}")
-        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype)
+        if (v is None or k.shape != (T, num_kv_heads * head_dim) or v.shape != (T, num_kv_heads * vd) or k.dtype != q.dtype
+                or v.dtype != q.dtype):
+            raise KernelError(f"rope: k / v must be [{T}, {num_kv_heads * head_dim}] / [{T}, {num_kv_heads * vd}] of {q.dtype}")
+        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype, vd)
         _i32(req_of_token, "req_of_token", T)
         if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
             raise KernelError("rope: block table must be contiguous int32 [requests, width]")
@@ -349,7 +367,7 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         _rows(v, "v") if write else 0, _dt(q), positions.data_ptr(), _ptr(req_of_token) if write else None,
         table_ptr, rdim, int(bool(inter)), T, num_heads, num_kv_heads, head_dim, int(write),
         _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, _ptr(block_table) if write else None,
-        block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0, 0, 0, _stream())
+        block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0, 0, 0, vd, _stream())
 
 
 def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_heads: int, num_kv_heads: int,
@@ -396,7 +414,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
                     block_table: torch.Tensor, ctx, num_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0, ws: Optional[KernelWorkspace] = None, *,
                     value_dim: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
-                    sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                    sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                    softcap: float = 0.0, out_scale: float = 1.0) -> None:
     """Causal attention of every token of the step over its request's pages.
 
     ``ctx`` carries ``positions`` and ``req_of_token`` ([T] int32), the step's shape on the host
@@ -406,12 +425,16 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     Options: ``value_dim`` (values of another width than keys; ``out`` is then [T, heads * value_dim]),
     ``slopes`` (float32 [heads]: slope * distance is taken off a key's scaled score), ``sinks``
     (float32 [heads]: exp(sink) joins the softmax's denominator once), ``gate`` (float32
-    [T, heads]: multiplies a head's output).
+    [T, heads]: multiplies a head's output), ``softcap`` (c > 0: the scaled score s becomes c * tanh(s / c)),
+    ``out_scale`` (a factor on every output, applied in float32 before the one rounding).
     """
     _gpu(out, q, k_cache, v_cache, block_table, ctx.positions, ctx.req_of_token)
     T = q.shape[0]
     vd = head_dim if value_dim is None else int(value_dim)
-    plain = vd == head_dim and slopes is None and sinks is None and gate is None
+    softcap, out_scale = float(softcap or 0.0), float(out_scale)
+    if softcap < 0.0:
+        raise KernelError(f"attention: a cap on the scores must be positive, got {softcap}")
+    plain = vd == head_dim and slopes is None and sinks is None and gate is None and softcap == 0.0 and out_scale == 1.0
     if plain:
         check_attention_sizes(num_heads, num_kv_heads, head_dim)
     else:
@@ -428,7 +451,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise KernelError("attention: block table must be contiguous int32 [requests, width]")
     if T == 0:
         return
-    if _FAST and q.dtype == torch.bfloat16 and vd == head_dim and head_dim % 16 == 0 and (plain or scale > 0):
+    if _FAST and q.dtype == torch.bfloat16 and vd == head_dim and head_dim % 16 == 0 and (plain or scale > 0) and softcap == 0.0 and out_scale == 1.0:
         # the matrix-core kernels take heads whose values are as wide as their keys, options included
         from . import fast
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
@@ -442,7 +465,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
               _rows(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), _dt(q), block_table.data_ptr(),
               block_table.shape[1], ctx.req_of_token.data_ptr(), ctx.positions.data_ptr(), T, num_heads,
               num_kv_heads, head_dim, page_size, float(scale), int(window), pages, ranges, _ptr(part),
-              0 if part is None else part.numel(), vd, _ptr(slopes), _ptr(sinks), _ptr(gate), _stream())
+              0 if part is None else part.numel(), vd, _ptr(slopes), _ptr(sinks), _ptr(gate), softcap, out_scale, _stream())
 
 
 def general_attention_ranges(tokens: int, num_heads: int, max_kv_len: int) -> int:
@@ -619,8 +642,9 @@ def matrix_memory_scan(out: torch.Tensor, proj: torch.Tensor, offsets, i_bias: t
               state.data_ptr(), state.shape[1], state.shape[0], heads, key_dim, value_dim, T, longest, _ptr(work), floats, _stream())
 
 
-def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, value_dim: int) -> None:
-    """y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gates[t, h, :])."""
+def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, value_dim: int,
+                   mult: float = 1.0) -> None:
+    """y[t, h, :] = mult * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gates[t, h, :])."""
     _gpu(y, o, gates, weight)
     T, N = y.shape[0], heads * value_dim
     if tuple(y.shape) != (T, N) or not y.is_contiguous():
@@ -630,7 +654,7 @@ def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight
             raise KernelError(f"head norm: {what} must be float32 [{T}, >= {N}]")
     _f32_vector(weight, N, "head norm weight")
     _lib.call("core", "pi_head_norm_gate", y.data_ptr(), _dt(y), o.data_ptr(), _rows(o, "o"), gates.data_ptr(), _rows(gates, "gates"),
-              weight.data_ptr(), float(eps), T, heads, value_dim, _stream())
+              weight.data_ptr(), float(eps), T, heads, value_dim, float(mult), _stream())
 
 
 # ----------------------------------------------------------------------------- routed experts
@@ -755,3 +779,126 @@ def combine_choices(out: torch.Tensor, y: torch.Tensor, weights: torch.Tensor, r
         raise KernelError("combine: one float32 weight per entry is needed")
     _lib.call("core", "pi_combine_choices", out.data_ptr(), y.data_ptr(), weights.data_ptr(), rows.entry_row.data_ptr(), T, rows.top, D,
               int(bool(accumulate)), _stream())
+
+
+# ----------------------------------------------------------------------------- mixers with a state of fixed size
+CONV_MAX_TAPS = 8
+
+
+def _state_rows(state: torch.Tensor, floats: int, what: str) -> None:
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < floats or not state.is_cuda:
+        raise KernelError(f"{what}: state must be float32 [slots, >= {floats}] with dense rows on the GPU, got {state.dtype} {tuple(state.shape)}")
+
+
+def _f32_rows(t: torch.Tensor, T: int, cols: int, what: str) -> int:
+    if t.dtype != torch.float32 or t.dim() != 2 or t.shape[0] != T or t.shape[1] < cols:
+        raise KernelError(f"{what}: expected float32 [{T}, >= {cols}], got {t.dtype} {tuple(t.shape)}")
+    return _rows(t, what)
+
+
+def causal_conv_silu(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], ctx,
+                     state: torch.Tensor) -> None:
+    """out[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - (taps - 1) + j, c]) within each request of the
+    step; the inputs before a request's first token of this step come from its state row
+    (``state`` float32 [slots, >= (taps - 1) * C], laid out [taps - 1, C], rows ``ctx.slots``), which
+    then takes the request's last taps - 1 inputs.  ``x`` and ``out`` are float32 [T, >= C] (column
+    views of wider tensors are fine; not in place)."""
+    _gpu(out, x, weight, bias, state)
+    T = x.shape[0]
+    C, taps = weight.shape
+    if taps > CONV_MAX_TAPS:
+        raise KernelError(f"convolution: {taps} taps are more than {CONV_MAX_TAPS}")
+    if not weight.is_contiguous() or (bias is not None and (bias.shape != (C,) or bias.dtype != weight.dtype or not bias.is_contiguous())):
+        raise KernelError(f"convolution: weight must be contiguous [{C}, {taps}] and bias [{C}] of the same type")
+    ldx, ldo = _f32_rows(x, T, C, "convolution input"), _f32_rows(out, T, C, "convolution output")
+    _state_rows(state, (taps - 1) * C, "convolution")
+    _i32(ctx.q_start, "q_start", ctx.R + 1)
+    _i32(ctx.slots, "slots", ctx.R)
+    longest = int(getattr(ctx, "max_q_len", 0) or T)
+    _lib.call("core", "pi_causal_conv_silu", out.data_ptr(), ldo, x.data_ptr(), ldx, weight.data_ptr(), _ptr(bias), _dt(weight), C, taps,
+              ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, longest, state.data_ptr(), state.stride(0), _stream())
+
+
+def state_space_scan(y: torch.Tensor, xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+                     skip: torch.Tensor, ctx, state: torch.Tensor, heads: int, value_dim: int, state_dim: int, groups: int) -> None:
+    """The state-space recurrence over the step's tokens, request by request, from and into the
+    requests' state rows (``state`` float32 [slots, >= heads * state_dim * value_dim], rows ``ctx.slots``):
+    ``S <- exp(-exp(a_log) * dt') S + dt' B x^T``, ``y = S^T C + skip * x`` with ``dt' = softplus(dt + dt_bias)``.
+    ``xbc`` float32 rows hold x [heads * value_dim], B and C [groups * state_dim each]; ``dt`` float32 [T, heads]
+    (a column view is fine); ``y`` float32 [T, heads * value_dim]."""
+    _gpu(y, xbc, dt, dt_bias, a_log, skip, state)
+    T, inner = y.shape[0], heads * value_dim
+    ldy = _f32_rows(y, T, inner, "state space output")
+    ldx = _f32_rows(xbc, T, inner + 2 * groups * state_dim, "state space input")
+    ldd = _f32_rows(dt, T, heads, "state space steps")
+    for t, what in ((dt_bias, "step bias"), (a_log, "decay"), (skip, "skip")):
+        _f32_vector(t, heads, f"state space {what}")
+    _state_rows(state, heads * state_dim * value_dim, "state space")
+    _i32(ctx.q_start, "q_start", ctx.R + 1)
+    _i32(ctx.slots, "slots", ctx.R)
+    _lib.call("core", "pi_state_space_scan", y.data_ptr(), ldy, xbc.data_ptr(), ldx, dt.data_ptr(), ldd, dt_bias.data_ptr(),
+              a_log.data_ptr(), skip.data_ptr(), ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, state.data_ptr(),
+              state.stride(0), heads, value_dim, state_dim, groups, _stream())
+
+
+def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, parts: int,
+                     mult: float = 1.0) -> None:
+    """out = mult * weight * v / sqrt(mean(v^2) + eps) with v = y * silu(z), the mean taken over each
+    of ``parts`` equal parts of a row.  ``y``, ``z`` float32 [T, >= N]; ``out`` [T, N] in any type."""
+    _gpu(out, y, z, weight)
+    T, N = out.shape
+    if N % parts:
+        raise KernelError(f"gated norm: {N} columns do not split into {parts} parts")
+    _f32_vector(weight, N, "gated norm weight")
+    _lib.call("core", "pi_gated_group_norm", out.data_ptr(), _dt(out), _rows(out, "gated norm out"), y.data_ptr(),
+              _f32_rows(y, T, N, "gated norm input"), z.data_ptr(), _f32_rows(z, T, N, "gated norm gate"), weight.data_ptr(),
+              float(eps), float(mult), T, N, int(parts), _stream())
+
+
+def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, b: torch.Tensor,
+               ctx, state: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int, q_scale: float,
+               unit_eps: float) -> None:
+    """The gated delta rule with a decay per head and key channel over the step's tokens, from and
+    into the requests' state rows (``state`` float32 [slots, >= heads * key_dim * value_dim]):
+    ``S <- diag(decay) S; u = beta (v - S^T k^); S <- S + k^ u^T; o = S^T q^`` with unit vectors
+    ``k^``, ``q^`` (the latter times ``q_scale``), ``decay = exp(-exp(a_log) * softplus(a + dt_bias))``,
+    ``beta = sigmoid(b)``.  ``qkv`` float32 rows hold q and k [kv_heads * key_dim each] and v
+    [heads * value_dim]; ``a`` float32 [T, heads * key_dim]; ``b`` float32 [T, heads] (a column view
+    is fine); ``o`` float32 [T, heads * value_dim]."""
+    _gpu(o, qkv, a, dt_bias, a_log, b, state)
+    T = o.shape[0]
+    ldo = _f32_rows(o, T, heads * value_dim, "delta rule output")
+    ldq = _f32_rows(qkv, T, 2 * kv_heads * key_dim + heads * value_dim, "delta rule input")
+    lda = _f32_rows(a, T, heads * key_dim, "delta rule decays")
+    ldb = _f32_rows(b, T, heads, "delta rule beta")
+    _f32_vector(dt_bias, heads * key_dim, "delta rule decay bias")
+    _f32_vector(a_log, heads, "delta rule decay rate")
+    _state_rows(state, heads * key_dim * value_dim, "delta rule")
+    _i32(ctx.q_start, "q_start", ctx.R + 1)
+    _i32(ctx.slots, "slots", ctx.R)
+    _lib.call("core", "pi_delta_scan", o.data_ptr(), ldo, qkv.data_ptr(), ldq, a.data_ptr(), lda, dt_bias.data_ptr(), a_log.data_ptr(),
+              b.data_ptr(), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, state.data_ptr(), state.stride(0), heads,
+              kv_heads, key_dim, value_dim, float(q_scale), float(unit_eps), _stream())
+
+
+def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, gate_bias: torch.Tensor, up_bias: torch.Tensor, limit: float,
+                alpha: float, x: Optional[torch.Tensor] = None, x_bias: Optional[torch.Tensor] = None) -> None:
+    """out = g * sigmoid(alpha * g) * (u + 1) with g = min(gate + gate_bias, limit) and
+    u = clamp(up + up_bias, -limit, limit); ``gate_up`` [T, 2I] holds the two products in halves.
+    With ``x`` (the float32 stream) and ``x_bias``: x[t, :] += x_bias as well, the bias of the product
+    that follows."""
+    _gpu(out, gate_up, gate_bias, up_bias, x, x_bias)
+    T, I = out.shape
+    if gate_up.shape != (T, 2 * I) or not (out.is_contiguous() and gate_up.is_contiguous()):
+        raise KernelError(f"clamped unit: expected contiguous gate_up [{T}, {2 * I}], got {tuple(gate_up.shape)}")
+    biases = [gate_bias, up_bias] + ([x_bias] if x is not None else [])
+    if any(b.dtype != gate_bias.dtype or not b.is_contiguous() for b in biases) or gate_bias.numel() != I or up_bias.numel() != I:
+        raise KernelError(f"clamped unit: biases must be contiguous [{I}] of one type")
+    D = 0
+    if x is not None:
+        D = x.shape[1]
+        if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[0] != T or x_bias is None or x_bias.numel() != D:
+            raise KernelError(f"clamped unit: the stream must be contiguous float32 [{T}, D] with a bias [D]")
+    _lib.call("core", "pi_clamped_glu", out.data_ptr(), _dt(out), gate_up.data_ptr(), _dt(gate_up), gate_bias.data_ptr(),
+              up_bias.data_ptr(), _ptr(x_bias) if x is not None else None, _dt(gate_bias), float(limit), float(alpha), T, I,
+              _ptr(x), D, _stream())

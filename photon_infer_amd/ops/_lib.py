@@ -16,16 +16,22 @@ P, I, L, F = c_void_p, c_int, c_long, c_float
 _SIGNATURES = {
     "core": {
         "pi_embedding": [P, P, I, P, I, I, I, P],
+        "pi_embedding_positions": [P, P, P, I, P, P, F, I, I, I, I, P],
+        "pi_clamped_glu": [P, I, P, I, P, P, P, I, F, F, I, I, P, I, P],
+        "pi_causal_conv_silu": [P, L, P, L, P, P, I, I, I, P, P, I, I, P, L, P],
+        "pi_state_space_scan": [P, L, P, L, P, L, P, P, P, P, P, I, P, L, I, I, I, I, P],
+        "pi_gated_group_norm": [P, I, L, P, L, P, L, P, F, F, I, I, I, P],
+        "pi_delta_scan": [P, L, P, L, P, L, P, P, P, L, P, P, I, P, L, I, I, I, I, F, F, P],
         "pi_rmsnorm": [P, I, P, P, P, I, F, I, I, P, I, L, P],
         "pi_swiglu": [P, P, I, I, I, I, P],
-        "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, P],
+        "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, I, P],
         "pi_gemm_general": [P, I, L, P, I, L, P, I, L, I, I, I, I, P],
-        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, P],
+        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, F, F, P],
         "pi_branch_norm_add": [P, P, I, P, P, P, P, P, F, F, I, I, P],
         "pi_cast_stream": [P, I, P, L, P],
         "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, L, P],
         "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, I, I, P, L, P],
-        "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, P],
+        "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, F, P],
         "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
         "pi_group_entries": [P, I, I, P, P, P, P, P, I, I, P],
         "pi_gather_rows": [P, P, I, P, I, I, I, P],

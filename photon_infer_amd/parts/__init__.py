@@ -7,10 +7,12 @@ from .rope import RotaryEmbedding, rope_frequencies
 from .attention import PagedAttention
 from .sink_attention import SinkWindowAttention
 from .matrix_memory import MatrixMemory
-from .mlp import SwiGLU
+from .state_space import StateSpaceMixer
+from .delta_rule import ChannelDeltaRule
+from .mlp import ClampedGLU, SwiGLU
 from .routed_experts import RoutedExperts
-from .block import OutputNormBlock, PreNormBlock
-from .embedding import LMHead, TokenEmbedding
+from .block import OutputNormBlock, PreNormBlock, SideBySide
+from .embedding import LMHead, PositionedEmbedding, TokenEmbedding
 from .model import CachePlan, DecoderModel, ModelSpec, RunEntry, plan_cache
 
 __all__ = [
@@ -18,5 +20,5 @@ __all__ = [
     "KVCacheSpec", "LayerCache", "Mixer", "Norm", "PAGE", "PagedCacheSpec", "PagedTensor", "Part", "PositionEncoding", "StateSpec",
     "StepContext", "RMSNorm", "RotaryEmbedding", "rope_frequencies", "PagedAttention", "SwiGLU",
     "PreNormBlock", "OutputNormBlock", "SinkWindowAttention", "MatrixMemory", "RoutedExperts", "LMHead", "TokenEmbedding", "CachePlan", "DecoderModel", "ModelSpec",
-    "RunEntry", "plan_cache",
+    "RunEntry", "plan_cache", "StateSpaceMixer", "ChannelDeltaRule", "ClampedGLU", "SideBySide", "PositionedEmbedding",
 ]

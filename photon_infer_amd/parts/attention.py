@@ -13,6 +13,12 @@ token carries its own position and sees only keys at positions <= its own, so a
 prompt may be cut into portions anywhere.
 
 An optional ``window`` W restricts a query at p to keys p-W+1..p.
+
+Further options, each a constructor parameter: values of another width than keys
+(``value_dim``), a cap on the scores (``softcap`` c: the scaled score s becomes
+``c * tanh(s / c)`` before the softmax), a factor on the mixer's result (``out_scale``, for
+arrangements that weigh mixers side by side; applied to the attention's float32 output before
+its one rounding, so that the output projection needs no second pass), and other tensor names.
 """
 from __future__ import annotations
 
@@ -23,7 +29,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import TensorSpec
-from .base import MIXERS, KVCacheSpec, LayerCache, Mixer, PositionEncoding, StepContext
+from .base import MIXERS, PAGE, KVCacheSpec, LayerCache, Mixer, PagedCacheSpec, PagedTensor, PositionEncoding, StepContext
 
 
 POSITION_PREFIX = "position."
@@ -40,6 +46,10 @@ class PagedAttention(Mixer):
         scale: Optional[float] = None,
         window: Optional[int] = None,
         own_kv: bool = True,
+        value_dim: Optional[int] = None,
+        softcap: Optional[float] = None,
+        out_scale: float = 1.0,
+        names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight"),
     ):
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
@@ -49,23 +59,37 @@ class PagedAttention(Mixer):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.window = int(window) if window else None
         self.own_kv = bool(own_kv)  # False: the layer has no k/v projection and reads another's cache
+        self.value_dim = int(value_dim) if value_dim else self.head_dim
+        self.softcap = float(softcap) if softcap else 0.0
+        self.out_scale = float(out_scale)
+        self.names = tuple(names)          # the q, k, v and o matrices' names after the part's prefix
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
-        ops.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
+        self.v_size = self.num_kv_heads * self.value_dim
+        self.o_size = self.num_heads * self.value_dim
+        # what only the general kernels and the separate rotation serve
+        self.with_options = self.value_dim != self.head_dim or self.softcap > 0.0 or self.out_scale != 1.0
+        if self.value_dim == self.head_dim:
+            ops.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
+        else:
+            ops.check_general_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim)
 
     def tensor_specs(self) -> List[TensorSpec]:
-        specs = [TensorSpec("q_proj.weight", (self.q_size, self.hidden_size))]
+        specs = [TensorSpec(self.names[0], (self.q_size, self.hidden_size))]
         if self.own_kv:
             specs += [
-                TensorSpec("k_proj.weight", (self.kv_size, self.hidden_size)),
-                TensorSpec("v_proj.weight", (self.kv_size, self.hidden_size)),
+                TensorSpec(self.names[1], (self.kv_size, self.hidden_size)),
+                TensorSpec(self.names[2], (self.v_size, self.hidden_size)),
             ]
-        specs.append(TensorSpec("o_proj.weight", (self.hidden_size, self.q_size)))
+        specs.append(TensorSpec(self.names[3], (self.hidden_size, self.o_size)))
         if self.position is not None:     # a position encoding with tensors of its own keeps them under "position."
             specs += [s.with_prefix(POSITION_PREFIX) for s in self.position.tensor_specs()]
         return specs
 
     def cache_spec(self):
+        if self.value_dim != self.head_dim:
+            return PagedCacheSpec((PagedTensor("k", (self.num_kv_heads, PAGE, self.head_dim)),
+                                   PagedTensor("v", (self.num_kv_heads, self.value_dim, PAGE))), self.window)
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
     @property
@@ -75,18 +99,20 @@ class PagedAttention(Mixer):
         return self.position is None or bool(self.position.graph_safe)
 
     def step_planner(self, page_size: int):
+        if self.value_dim != self.head_dim:      # only the general kernel takes such heads; it needs no work lists
+            return None
         return ops.attention_planner(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim, page_size,
                                      self.window or 0, self.device)
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
-        mats = [tensors["q_proj.weight"]]
+        mats = [tensors[self.names[0]]]
         if self.own_kv:
-            mats += [tensors["k_proj.weight"], tensors["v_proj.weight"]]
+            mats += [tensors[self.names[1]], tensors[self.names[2]]]
         # one projection for q, k and v: rows [q heads | k heads | v heads]
         common = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
         self.w_qkv = torch.cat([m.to(common) for m in mats], dim=0).contiguous()
-        self.w_o = tensors["o_proj.weight"]
+        self.w_o = tensors[self.names[3]]
         if self.position is not None:
             own = {n[len(POSITION_PREFIX):]: t for n, t in tensors.items() if n.startswith(POSITION_PREFIX)}
             self.position.load(own, dtype, device)
@@ -102,7 +128,7 @@ class PagedAttention(Mixer):
         table = ctx.block_tables[cache.group]
         ws = ctx.workspace
         qkv = ops.qkv_projection(h, self.w_qkv, self.dtype, ws) if fused_position else None
-        if qkv is not None and ctx.all_decode:
+        if qkv is not None and ctx.all_decode and not self.with_options:
             # single tokens only: one kernel rotates, writes the cache and attends
             attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
             done = ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
@@ -118,7 +144,7 @@ class PagedAttention(Mixer):
             q = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
             ops.rope_kv_write(q, None, None, ctx.positions, ctx.req_of_token, rotary, self.num_heads,
                               self.num_kv_heads, self.head_dim, cache.k, cache.v, table, cache.page_size,
-                              pieces=qkv, write_kv=writes)
+                              pieces=qkv, write_kv=writes, value_dim=self.value_dim)
         else:
             if qkv is None:
                 qkv = torch.empty((T, self.w_qkv.shape[0]), dtype=self.dtype, device=h.device)
@@ -131,13 +157,19 @@ class PagedAttention(Mixer):
             ops.rope_kv_write(
                 q, k if writes else None, v if writes else None, ctx.positions, ctx.req_of_token,
                 rotary, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v, table, cache.page_size,
+                value_dim=self.value_dim,
             )
-        attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
-        ops.paged_attention(
-            attn, q, cache.k, cache.v, table, ctx,
-            self.num_heads, self.num_kv_heads, self.head_dim, cache.page_size,
-            self.scale, self.window or 0, ws,
-        )
+        attn = torch.empty((T, self.o_size), dtype=self.dtype, device=h.device)
+        if self.with_options:
+            ops.paged_attention(attn, q, cache.k, cache.v, table, ctx, self.num_heads, self.num_kv_heads, self.head_dim,
+                                cache.page_size, self.scale, self.window or 0, ws, value_dim=self.value_dim,
+                                softcap=self.softcap, out_scale=self.out_scale)
+        else:
+            ops.paged_attention(
+                attn, q, cache.k, cache.v, table, ctx,
+                self.num_heads, self.num_kv_heads, self.head_dim, cache.page_size,
+                self.scale, self.window or 0, ws,
+            )
         # where the arrangement allows it, the product stays in pieces for the stream's next reader
         ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
 

@@ -6,31 +6,87 @@ src/arch/transformer_block.cpp:189-299):
 """
 from __future__ import annotations
 
-from typing import Dict, List, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
 from .. import ops
 from ..errors import UnsupportedModelError
 from ..weights.loader import TensorSpec
-from .base import BLOCKS, Block, FeedForward, LayerCache, Mixer, Norm, Part, StepContext
+from .base import BLOCKS, MIXERS, Block, FeedForward, LayerCache, Mixer, Norm, Part, StepContext
+
+
+class SideBySide(Mixer):
+    """Several mixers that read the same input, their results summed into the stream:
+    ``x += sum_i scale_i * mixer_i(h)``.  Every mixer keeps a cache or state of its own
+    (``mixers()``; ``forward`` takes their ``LayerCache`` in that order) and applies its own
+    factor (its ``out_scale``) to its last activation, in float32, before the output projection
+    that accumulates into the stream: the sum costs no kernel.
+
+    ``branches``: [(prefix, mixer)]."""
+
+    def __init__(self, branches):
+        if not branches:
+            raise UnsupportedModelError("mixers side by side: none given")
+        self.branches: List[Tuple[str, Mixer]] = list(branches)
+        for _, m in self.branches:
+            if not getattr(m, "accumulate", True):
+                raise UnsupportedModelError(f"{type(m).__name__} must add its result into the stream to stand beside other mixers")
+
+    def mixers(self) -> List[Mixer]:
+        return [m for _, m in self.branches]
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s.with_prefix(p) for p, m in self.branches for s in m.tensor_specs()]
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        for prefix, m in self.branches:
+            names = [prefix + s.name for s in m.tensor_specs()]
+            m.load({n[len(prefix):]: tensors[n] for n in names}, dtype, device)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(m.graph_safe for _, m in self.branches)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for _, m in self.branches for w in m.streamed_weights()]
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache) -> None:
+        caches = cache if isinstance(cache, (list, tuple)) else [cache]
+        for (_, m), c in zip(self.branches, caches):
+            m.forward(h, x, ctx, c)
+
+
+MIXERS.register("side_by_side", SideBySide)
 
 
 class PreNormBlock(Block):
-    """Each of the four parts comes with the name prefix of its tensors inside the block."""
+    """Each of the four parts comes with the name prefix of its tensors inside the block.  The
+    mixer may be several side by side (``SideBySide``); ``norm2`` and ``ffn`` None: a layer without
+    a feed-forward."""
 
     def __init__(self, norm1: Tuple[str, Norm], mixer: Tuple[str, Mixer],
-                 norm2: Tuple[str, Norm], ffn: Tuple[str, FeedForward]):
-        self._named: List[Tuple[str, Part]] = [norm1, mixer, norm2, ffn]
-        self.norm1, self.mixer, self.norm2, self.ffn = norm1[1], mixer[1], norm2[1], ffn[1]
+                 norm2: Optional[Tuple[str, Norm]] = None, ffn: Optional[Tuple[str, FeedForward]] = None):
+        if (ffn is None) != (norm2 is None):
+            raise UnsupportedModelError("a feed-forward and its norm come together")
+        self._named: List[Tuple[str, Part]] = [norm1, mixer] + ([norm2, ffn] if ffn is not None else [])
+        self.norm1, self.mixer = norm1[1], mixer[1]
+        self.norm2, self.ffn = (norm2[1], ffn[1]) if ffn is not None else (None, None)
+
+    def mixers(self) -> List[Mixer]:
+        inner = getattr(self.mixer, "mixers", None)
+        return inner() if inner is not None else [self.mixer]
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [s.with_prefix(p) for p, part in self._named for s in part.tensor_specs()]
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
+        # a part's tensors: those named by its own list (a prefix may be a prefix of another)
         for prefix, part in self._named:
-            part.load({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, dtype, device)
+            names = [prefix + s.name for s in part.tensor_specs()]
+            part.load({n[len(prefix):]: tensors[n] for n in names}, dtype, device)
 
     @property
     def graph_safe(self) -> bool:
@@ -47,6 +103,11 @@ class PreNormBlock(Block):
         # A mixer or feed-forward may leave its update of x in pieces (ops.gemm(..., may_defer=True))
         # when the stream's next reader adds them: norm2 after the mixer; after the feed-forward,
         # whoever the model says reads the stream next.
+        if self.ffn is None:
+            ctx.may_defer = ctx.after_block_consumes
+            self.mixer.forward(self.norm1.forward(x, ctx), x, ctx, cache)
+            ctx.may_defer = False
+            return
         ctx.may_defer = bool(getattr(self.norm2, "consumes_deferred", False))
         self.mixer.forward(self.norm1.forward(x, ctx), x, ctx, cache)
         ctx.may_defer = ctx.after_block_consumes

@@ -32,11 +32,47 @@ class TokenEmbedding(Part):
         super().load(tensors, dtype, device)
         self.weight = tensors[self.tensor_name]
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        """int32 [T] -> float32 residual stream [T, hidden]."""
+    def forward(self, token_ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        """int32 [T] -> float32 residual stream [T, hidden].  ``ctx``: the step's context, for
+        embeddings that look at more than the ids."""
         x = torch.empty((token_ids.shape[0], self.hidden_size), dtype=torch.float32, device=token_ids.device)
         ops.embedding(x, self.weight, token_ids)
         return x
+
+
+class PositionedEmbedding(TokenEmbedding):
+    """``x = norm(table[token] * scale + positions[p])``: a scaled embedding, a learned vector per
+    absolute position (not scaled; the table's rows bound the sequence length), and a norm of the
+    sum, whose float32 result is the residual stream.  ``norm`` = (tensor name prefix, Norm) or None."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, max_positions: int, scale: float = 1.0, norm=None,
+                 tensor_name: str = "weight", position_name: str = "positions"):
+        super().__init__(vocab_size, hidden_size, tensor_name)
+        self.max_positions, self.scale = int(max_positions), float(scale)
+        self.position_name = position_name
+        self.norm_prefix, self.norm = norm if norm is not None else ("", None)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = super().tensor_specs() + [TensorSpec(self.position_name, (self.max_positions, self.hidden_size), "table")]
+        if self.norm is not None:
+            specs += [s.with_prefix(self.norm_prefix) for s in self.norm.tensor_specs()]
+        return specs
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        self.positions = tensors[self.position_name].to(self.weight.dtype)
+        if self.norm is not None:
+            names = [self.norm_prefix + s.name for s in self.norm.tensor_specs()]
+            self.norm.load({n[len(self.norm_prefix):]: tensors[n] for n in names}, dtype, device)
+
+    def forward(self, token_ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        x = torch.empty((token_ids.shape[0], self.hidden_size), dtype=torch.float32, device=token_ids.device)
+        ops.embedding(x, self.weight, token_ids, self.scale, self.positions, ctx.positions)
+        if self.norm is None:
+            return x
+        out = torch.empty_like(x)
+        ops.rmsnorm(out, x, self.norm.weight, self.norm.eps)
+        return out
 
 
 class LMHead(Part):

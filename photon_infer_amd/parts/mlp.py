@@ -72,3 +72,55 @@ class SwiGLU(FeedForward):
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)
+
+
+class ClampedGLU(FeedForward):
+    """A gated feed-forward with biases, clamped before the gate's activation:
+
+        g = min(W_gate h + b_gate, limit);  u = clamp(W_up h + b_up, -limit, limit)
+        y = g * sigmoid(alpha * g) * (u + 1);  x += W_down y + b_down
+
+    ``limit`` and ``alpha`` are parameters.  Biases are added and the unit is computed in float32
+    from the float32 results of the one gate | up product; the down projection's bias joins the
+    stream in the same kernel, so that the product only accumulates."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702,
+                 names=("gate", "up", "down"), bias_suffix: str = ".b"):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.names, self.bias_suffix = tuple(names), bias_suffix
+        self.accumulate = True           # adds into the stream; there is no writing form
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        I, D, b = self.intermediate_size, self.hidden_size, self.bias_suffix
+        g, u, d = self.names
+        return [TensorSpec(g, (I, D)), TensorSpec(g + b, (I,), "small_bias"), TensorSpec(u, (I, D)), TensorSpec(u + b, (I,), "small_bias"),
+                TensorSpec(d, (D, I)), TensorSpec(d + b, (D,), "small_bias")]
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        g, u, d = self.names
+        wg, wu = tensors[g], tensors[u]
+        common = torch.float32 if torch.float32 in (wg.dtype, wu.dtype) else wg.dtype
+        self.w_gate_up = torch.cat([wg.to(common), wu.to(common)], dim=0).contiguous()       # rows [gate | up]
+        self.w_down = tensors[d]
+        f32 = lambda t: t.to(torch.float32).contiguous()
+        self.b_gate, self.b_up, self.b_down = f32(tensors[g + self.bias_suffix]), f32(tensors[u + self.bias_suffix]), f32(tensors[d + self.bias_suffix])
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_gate_up, self.w_down]
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        T, I = h.shape[0], self.intermediate_size
+        ws = ctx.workspace if ctx is not None else None
+        gu = torch.empty((T, 2 * I), dtype=torch.float32, device=h.device)
+        ops.gemm(gu, h, self.w_gate_up, ws=ws)
+        act = torch.empty((T, I), dtype=self.dtype, device=h.device)
+        ops.materialize(x, ws)          # the bias is added to the stream itself
+        ops.clamped_glu(act, gu, self.b_gate, self.b_up, self.limit, self.alpha, x, self.b_down)
+        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
+
+
+FEED_FORWARDS.register("clamped_glu", ClampedGLU)

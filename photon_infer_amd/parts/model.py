@@ -148,7 +148,7 @@ class DecoderModel:
         ws = ctx.workspace
         ops.reset_deferred(ws)             # nothing of an earlier (failed) step may linger
         ctx.scratch.clear()
-        x = self.embedding.forward(ctx.token_ids)
+        x = self.embedding.forward(ctx.token_ids, ctx)
         order = self.spec.run_order
         wanted = ctx.logit_rows.shape[0] > 0
         for i, entry in enumerate(order):

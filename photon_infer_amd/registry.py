@@ -67,7 +67,13 @@ def config_from_dict(raw: dict, where: str = "config.json"):
 def load_config(model_dir: str):
     """Read ``model_dir/config.json`` into the typed config of its architecture."""
     raw = read_config_json(model_dir)
-    return config_from_dict(raw, f"{model_dir}/config.json")
+    config = config_from_dict(raw, f"{model_dir}/config.json")
+    # a design may leave sizes to the tensors' shapes; the folder's headers are read only if it asks
+    complete = getattr(config, "with_tensor_shapes", None)
+    if complete is not None:
+        from .weights.safetensors_io import tensor_shapes
+        config = complete(lambda: tensor_shapes(model_dir))
+    return config
 
 
 def build_model_spec(config):

@@ -40,6 +40,10 @@ def random_tensors(specs: Iterable[TensorSpec], seed: int, std: float = 0.02, no
             t = torch.zeros(s.shape) if norm_init == "ones" else torch.rand(s.shape, generator=g) - 0.5
         elif s.role == "bias":           # per-head numbers of order one (gate biases, sinks)
             t = torch.randn(s.shape, generator=g, dtype=torch.float32)
+        elif s.role == "small_bias":     # biases of projections and convolutions
+            t = torch.randn(s.shape, generator=g, dtype=torch.float32) * 0.1
+        elif s.role == "taps":           # a short convolution's weights: of order one, so that earlier inputs count
+            t = torch.randn(s.shape, generator=g, dtype=torch.float32) * 0.5
         elif s.role == "int_table":
             out[s.name] = torch.randint(0, 2**15, s.shape, generator=g, dtype=torch.int32)
             continue

@@ -164,3 +164,16 @@ def open_model_files(model_dir: str) -> list:
         f"model folder '{model_dir}' has neither model.safetensors nor model.safetensors.index.json",
         ErrorCode.FILE_NOT_FOUND,
     )
+
+
+def tensor_shapes(model_dir: str) -> dict:
+    """name -> shape of every tensor in a model folder's weight files (headers only; no file: empty)."""
+    try:
+        files = open_model_files(model_dir)
+    except FileFormatError:
+        return {}
+    try:
+        return {n: tuple(f.entries[n].shape) for f in files for n in f.names()}
+    finally:
+        for f in files:
+            f.close()
