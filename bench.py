@@ -1,7 +1,7 @@
 #!/usr/bin/python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra|rorevik]
                     [--batch 8,1,64] [--context 4096] [--dtype bf16|fp32]
 
 Every workload prints ONE JSON line.  The default, ``decode1b`` (Llama 3.2 1B layer sizes):  ``value`` is decoded tokens per second at batch 8 with the context
@@ -40,6 +40,10 @@ mixed step, and the step's flops and bytes against the peaks.
 routed feed-forwards) at layer sizes like Llama 3.2 1B's and 3B's, beside a Llama of the same width,
 depth and vocabulary: a 2,048-token prompt and decode steps at batch 8, both through the same step
 functions.  ``value`` is Dafidra's decoded tokens per second at the first size.
+
+``--workload rorevik``: the Rorevik design (attention with capped scores beside a state-space mixer, a
+delta-rule memory in every third layer, clamped gated feed-forwards with biases) at layer sizes like
+Llama 3.2 1B's and 3B's, beside a Llama of the same width, depth and vocabulary, measured the same way.
 
 Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
 """
@@ -512,6 +516,75 @@ def workload_dafidra(args) -> int:
     return 0
 
 
+def rorevik_config(width, heads, kv_heads, head_dim, ff, vocab, layers, positions):
+    """A Rorevik of Llama-like layer sizes: attention as the Llama's (half of each head rotated, scores capped at 30),
+    beside it a state-space mixer as wide as the model (heads of 64, a state of 128, one group); every third layer
+    holds a delta-rule memory instead (heads of 128 keys and 128 values, as wide as the model, low-rank sizes 128);
+    clamped gated feed-forwards of the Llama's width with biases."""
+    left = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5, softcap=30.0,
+                rot={"base": 500000.0, "dims": head_dim // 2})
+    right = dict(heads=width // 64, vdim=64, state=128, groups=1, norm_groups=1, conv=4)
+    delta = dict(heads=width // 128, kv_heads=width // 128, dim=128, vdim=128, conv=4, decay_rank=128, gate_rank=128)
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    par = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp}
+    dlt = {"type": "channel_delta", "mixer": delta, "mlp": mlp}
+    return {"architecture": "Rorevik", "vocab": vocab, "width": width, "max_positions": positions, "embedding": {"scale": width ** 0.5},
+            "norm": {"eps": 1e-5}, "layers": [dlt if i % 3 == 2 else par for i in range(layers)]}
+
+
+def workload_rorevik(args) -> int:
+    """Rorevik beside a Llama of equal width, depth and vocabulary (see the module text)."""
+    import gc
+
+    import torch
+
+    layers = args.layers or 4
+    context = args.context
+    positions = max(context, PREFILL_TOKENS) + 64
+    sizes = {"1b": MODEL, "3b": MODEL_3B}
+    results = {}
+
+    def config(b):
+        return rorevik_config(b["hidden_size"], b["num_attention_heads"], b["num_key_value_heads"], b["head_dim"],
+                              b["intermediate_size"], b["vocab_size"], layers, positions)
+
+    if args.only:       # for profiles: the Rorevik of the first size alone, a prompt or decode steps
+        runner, _cfg = make_runner(config(sizes["1b"]), layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                   max_model_len=positions)
+        if args.only == "prefill":
+            sec = time_prefill(runner, PREFILL_TOKENS, max(1, args.steps // 8))
+            print(json.dumps({"only": "prefill", "model": "rorevik_1b", "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3)}), flush=True)
+        else:
+            sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context, synthetic_cache=True)
+            print(json.dumps({"only": "decode", "model": "rorevik_1b", "batch": args.batch, "ms_per_step": round(sec * 1e3, 4),
+                              "cache": "random numbers, no prompt was run"}), flush=True)
+        return 0
+    for name, base in sizes.items():
+        for what, raw in (("rorevik", config(base)), ("llama", dict(base, tie_word_embeddings=False))):
+            runner, _cfg = make_runner(raw, layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                       max_model_len=positions)
+            psec = time_prefill(runner, PREFILL_TOKENS, 3)
+            dsec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context)
+            results[f"{what}_{name}"] = {"prefill_ms": round(psec * 1e3, 3), "prefill_tok_per_s": round(PREFILL_TOKENS / psec, 1),
+                                         "decode_ms_per_step": round(dsec * 1e3, 4), "decode_tok_per_s": round(args.batch / dsec, 1),
+                                         "graphs": len(runner._graphs)}
+            del runner
+            gc.collect()
+            torch.cuda.empty_cache()
+    first = results["rorevik_1b"]
+    line = {
+        "metric": f"decode tok/s at batch {args.batch}, context {context} (Rorevik at Llama 3.2 1B layer sizes, {layers} layers, random weights)",
+        "value": first["decode_tok_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "rorevik-at-llama-sizes", "layers": layers, "global_batch": args.batch, "seq_len": context,
+                   "prefill_tokens": PREFILL_TOKENS, "kv_block": BLOCK_SIZE, "parallelism": "single-gpu"},
+        "models": results,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -520,7 +593,7 @@ def main() -> int:
     ap.add_argument("--batch", default="8,1,64",
                     help="batch sizes of the decode steps: the first is the headline's, the others become points")
     ap.add_argument("--context", type=int, default=CONTEXT, help="context length that the decode steps end at")
-    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra"], default="decode1b")
+    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra", "rorevik"], default="decode1b")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -554,6 +627,8 @@ def main() -> int:
         return workload_mixed8b(args)
     if args.workload == "dafidra":
         return workload_dafidra(args)
+    if args.workload == "rorevik":
+        return workload_rorevik(args)
     args.layers = args.layers or MODEL["num_hidden_layers"]
     elem = 2 if args.dtype == "bf16" else 4
     big = args.batch if (args.no_points or args.only) else max(batches)

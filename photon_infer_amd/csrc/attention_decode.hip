@@ -195,6 +195,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   st.pos[0] = p;
   st.lo[0] = lo;
   st.bias[0] = (OPT && valid && opt.slopes) ? opt.slopes[g * G + lr] / scale : 0.f;
+  attn_set_cap(st, OPT ? opt.softcap : 0.f, scale);
   // this wave's keys: chunk `split` of the 32-key chunks between lo and p
   const int first_chunk = lo / 32, last_chunk = p / 32;
   const int chunks = last_chunk - first_chunk + 1;
@@ -230,6 +231,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
       if (OPT) {
         if (opt.sinks) inv = sink_inverse(st.l[0], st.m[0] * (scale * PI_LOG2E), opt.sinks[head]);
         if (opt.gate) inv *= opt.gate[row * nh + head];
+        inv *= opt.out_mult;
       }
 #pragma unroll
       for (int db = 0; db < HD / 16; ++db) {
@@ -310,7 +312,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
   const long out_row = rows ? rows[blockIdx.y] : q_start[r];
   combine_ranges<HD>(out + out_row * out_stride + (long)head * HD, part + ((long)blockIdx.y * nh + head) * splits * (HD + 4),
                      splits, threadIdx.x, opt.sinks ? opt.sinks[head] * PI_LOG2E : -INFINITY,
-                     opt.gate ? opt.gate[out_row * nh + head] : 1.0f);
+                     (opt.gate ? opt.gate[out_row * nh + head] : 1.0f) * opt.out_mult);
 }
 
 // One wave per (row of `part`, head): rows are a launch's requests (results to the requests'
@@ -351,7 +353,7 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
                          const int* q_start, const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd,
                          int page_size, float scale, int window, long num_pages, int splits, void* part, long part_elems,
                          bool merge, hipStream_t stream, AttnOptions opt = AttnOptions{nullptr, nullptr, nullptr}) {
-  const bool with_options = opt.slopes || opt.sinks || opt.gate;
+  const bool with_options = opt.any();
   PI_REQUIRE(!with_options || (!fused && merge && scale > 0.f), "attention_decode: heads with options take the separate kernels, merged here, and a positive scale");
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
   PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_decode: head_dim %d is not a multiple of 16 up to 256", hd);
@@ -422,10 +424,11 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
                                    const void* v_cache, const int* block_table, int table_width, const int* q_start,
                                    const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd, int page_size,
                                    float scale, int window, long num_pages, int splits, void* part, long part_elems,
-                                   const float* slopes, const float* sinks, const float* gate, hipStream_t stream) {
+                                   const float* slopes, const float* sinks, const float* gate, float softcap, float out_mult,
+                                   hipStream_t stream) {
   return launch_decode(false, DecodeSource{}, out, out_stride, q, q_stride, k_cache, v_cache, block_table, table_width, q_start,
                        kv_len, req_ids, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, true, stream,
-                       AttnOptions{slopes, sinks, gate});
+                       AttnOptions{slopes, sinks, gate, softcap, out_mult});
 }
 
 // The same for a step of single tokens only (T == R tokens, request r at row q_start[r]),
@@ -474,7 +477,7 @@ extern "C" int pi_attention_decode_fused(void* out, long out_stride, const void*
 // Merge partial results that the tile kernel wrote for `Z` tokens whose tiles' keys were cut in
 // `cuts` shares: part [Z, nh, cuts, hd + 4]; token z's result goes to row rows[z] of out.
 extern "C" int pi_attention_combine_rows(void* out, long out_stride, const int* rows, int Z, const void* part, int nh, int hd,
-                                         int cuts, const float* sinks, const float* gate, hipStream_t stream) {
+                                         int cuts, const float* sinks, const float* gate, float out_mult, hipStream_t stream) {
   PI_REQUIRE(Z > 0 && Z <= 65535 && nh > 0 && cuts >= 2 && cuts <= 64 && rows && part, "attention_combine_rows: bad arguments (%d tokens, %d heads, %d cuts)", Z, nh, cuts);
-  return launch_combine(out, out_stride, nullptr, nullptr, rows, Z, part, nh, hd, cuts, stream, AttnOptions{nullptr, sinks, gate});
+  return launch_combine(out, out_stride, nullptr, nullptr, rows, Z, part, nh, hd, cuts, stream, AttnOptions{nullptr, sinks, gate, 0.f, out_mult});
 }

@@ -46,17 +46,37 @@ struct AttnState {
   int lo[CB];           // first visible key of the column
   float bias[CB];       // distance bias of the column's head per key of distance, in raw score units
                         // (slope / scale); read only by the BIAS variants of the arithmetic
+  float cap_raw;        // the cap on the scores in raw score units (cap / scale; 0: none), the same for every
+  float cap_rate;       // column; and 2 log2(e) scale / cap.  Read only by the BIAS variants.
 };
 
 // Options of a head beyond plain softmax attention, each off when its pointer is null:
 //   slopes [heads]: slope * (p - t) is taken off the scaled score of key t for the query at p;
 //   sinks  [heads]: exp(sink) joins the softmax's denominator once (no key, no value, no scale, no bias);
-//   gate   [tokens, heads] float32: multiplies the head's output.
+//   gate   [tokens, heads] float32: multiplies the head's output;
+//   softcap > 0: the scaled score s becomes softcap * tanh(s / softcap), before any bias;
+//   out_mult: a factor on every output.
 struct AttnOptions {
   const float* slopes;
   const float* sinks;
   const float* gate;
+  float softcap = 0.f;
+  float out_mult = 1.f;
+  bool any() const { return slopes || sinks || gate || softcap > 0.f || out_mult != 1.f; }
 };
+
+// A raw score r (before the softmax scale) capped: (cap / scale) * tanh(r * scale / cap), with
+// tanh(x) = 1 - 2 / (1 + e^2x) from one v_exp_f32 and one v_rcp_f32; +-inf end at +-cap.
+__device__ inline float capped_raw(float r, float cap_raw, float cap_rate) {
+  const float e = __builtin_amdgcn_exp2f(r * cap_rate);
+  return __builtin_fmaf(-2.0f * cap_raw, __builtin_amdgcn_rcpf(1.0f + e), cap_raw);
+}
+
+template <class State>
+__device__ inline void attn_set_cap(State& st, float softcap, float scale) {
+  st.cap_raw = softcap > 0.f ? softcap / scale : 0.f;
+  st.cap_rate = softcap > 0.f ? 2.0f * PI_LOG2E * scale / softcap : 0.f;
+}
 
 // The sink joins a column's sum of weights l, which is relative to the base-2 reference m2
 // (-inf: nothing seen): returns the factor for the un-normalised output, 1 / (l' ) included.
@@ -223,7 +243,11 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
       f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < HeadFrags<HD>::KS; ++ks) acc = mfma16(kv.key(t, ks), st.q[c][ks], acc);
-      if (BIAS) {   // the distance bias joins the raw score before anything looks at it
+      if (BIAS) {   // the cap, then the distance bias, join the raw score before anything looks at it
+        if (st.cap_raw != 0.f) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] = capped_raw(acc[i], st.cap_raw, st.cap_rate);
+        }
         const float base = st.bias[c] * (float)(k0 + t * 16 + lg * 4 - st.pos[c]);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] += __builtin_fmaf(st.bias[c], (float)i, base);
@@ -332,6 +356,16 @@ __device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* 
     __builtin_amdgcn_sched_group_barrier(0x008, KF * CB, 0);               // this chunk's products
   }
   if (BIAS) {
+    if (st.cap_raw != 0.f) {
+#pragma unroll
+      for (int c = 0; c < CB; ++c)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[j][t][c][i] = capped_raw(s[j][t][c][i], st.cap_raw, st.cap_rate);
+    }
 #pragma unroll
     for (int c = 0; c < CB; ++c) {
       const float base = st.bias[c] * (float)(key0 + (lane / 16) * 4 - st.pos[c]);

@@ -78,6 +78,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
 
     AttnState<HD, CB> st;
     attn_init(st);
+    attn_set_cap(st, OPT ? opt.softcap : 0.f, scale);
     long rows[CB];
     int heads[CB];
     bool valid[CB];
@@ -183,6 +184,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
       if (OPT) {
         if (opt.sinks) inv = sink_inverse(st.l[c], st.m[c] * scale_log2, opt.sinks[heads[c]]);
         if (opt.gate) inv *= opt.gate[rows[c] * nh + heads[c]];
+        inv *= opt.out_mult;
       }
       bf16_t* o = out + rows[c] * out_stride + (long)heads[c] * HD + lg * 4;
 #pragma unroll
@@ -215,7 +217,8 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
                                          const int* kv_len, const int* tile_req, const int* tile_q0, const int* tile_cut,
                                          const int* tile_z0, void* part, const int* order, int rounds, int seats, int nh,
                                          int nkv, int hd, int page_size, float scale, int window, long num_pages,
-                                         const float* slopes, const float* sinks, const float* gate, hipStream_t stream) {
+                                         const float* slopes, const float* sinks, const float* gate, float softcap,
+                                         float out_mult, hipStream_t stream) {
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
   PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_prefill: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
@@ -226,9 +229,9 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
   const dim3 grid(nkv, seats), block(256);
-  const AttnOptions opt{slopes, sinks, gate};
-  const bool with_options = slopes || sinks || gate;
-  PI_REQUIRE(!with_options || scale > 0.f, "attention_prefill: a distance bias needs a positive scale");
+  const AttnOptions opt{slopes, sinks, gate, softcap, out_mult};
+  const bool with_options = opt.any();
+  PI_REQUIRE(!with_options || scale > 0.f, "attention_prefill: a distance bias or a cap needs a positive scale");
 #define GO(H, C, N)                    \
   do {                                 \
     if (with_options) GO1(H, C, N, true); \

@@ -32,7 +32,7 @@ def _mixer(cfg: RorevikConfig, m):
         if a.rot_dims:
             rope = POSITION_ENCODINGS.make("rope", head_dim=a.dim, theta=a.rot_base, interleaved=True, rotary_dim=a.rot_dims)
         left = MIXERS.make("attention", hidden_size=D, num_heads=a.heads, num_kv_heads=a.kv_heads, head_dim=a.dim, position=rope,
-                           scale=a.scale, value_dim=a.vdim, softcap=a.softcap, out_scale=m.left_scale, names=("q", "k", "v", "o"))
+                           scale=a.scale, value_dim=a.vdim, softcap=a.softcap, out_scale=m.left_scale, names=("q", "k", "v", "o"), any_head_size=True)
         right = MIXERS.make("state_space", hidden_size=D, num_heads=r.heads, value_dim=r.vdim, state_dim=r.state, groups=r.groups,
                             norm_groups=r.norm_groups, conv_taps=r.conv, eps=eps, out_scale=m.right_scale)
         return MIXERS.make("side_by_side", branches=[("left.", left), ("right.", right)])

@@ -328,7 +328,7 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     _gpu(q, k, v, positions, req_of_token, k_cache, v_cache, block_table)
     T = q.shape[0]
     vd = head_dim if value_dim is None else int(value_dim)
-    if vd == head_dim:
+    if value_dim is None:
         check_attention_sizes(num_heads, num_kv_heads, head_dim)
     else:
         check_general_attention_sizes(num_heads, num_kv_heads, head_dim, vd)
@@ -434,7 +434,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     softcap, out_scale = float(softcap or 0.0), float(out_scale)
     if softcap < 0.0:
         raise KernelError(f"attention: a cap on the scores must be positive, got {softcap}")
-    plain = vd == head_dim and slopes is None and sinks is None and gate is None and softcap == 0.0 and out_scale == 1.0
+    plain = value_dim is None and slopes is None and sinks is None and gate is None and softcap == 0.0 and out_scale == 1.0
     if plain:
         check_attention_sizes(num_heads, num_kv_heads, head_dim)
     else:
@@ -451,11 +451,11 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise KernelError("attention: block table must be contiguous int32 [requests, width]")
     if T == 0:
         return
-    if _FAST and q.dtype == torch.bfloat16 and vd == head_dim and head_dim % 16 == 0 and (plain or scale > 0) and softcap == 0.0 and out_scale == 1.0:
+    if _FAST and q.dtype == torch.bfloat16 and vd == head_dim and head_dim % 16 == 0 and (plain or scale > 0):
         # the matrix-core kernels take heads whose values are as wide as their keys, options included
         from . import fast
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                                page_size, scale, window, pages, ws, slopes, sinks, gate):
+                                page_size, scale, window, pages, ws, slopes, sinks, gate, softcap, out_scale):
             return
     # a step of few tokens over long contexts: its keys cut into ranges, merged by a second kernel
     # (as many as the context-length bucket asks for, so that a step gives the same bits eagerly and replayed)

@@ -499,10 +499,12 @@ def _decode_splits_that_fit(ws, n_req: int, num_heads: int, num_kv_heads: int, h
 
 
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                    page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None, slopes=None, sinks=None, gate=None) -> bool:
+                    page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None, slopes=None, sinks=None, gate=None,
+                    softcap: float = 0.0, out_scale: float = 1.0) -> bool:
     """``slopes`` / ``sinks`` (float32 [heads]) and ``gate`` (float32 [tokens, heads]): a distance bias, a sink in
-    the softmax and an output gate per head (None: none)."""
-    opt = tuple(None if t is None else t.data_ptr() for t in (slopes, sinks, gate))
+    the softmax and an output gate per head (None: none); ``softcap`` > 0: scaled scores s become
+    softcap * tanh(s / softcap); ``out_scale``: a factor on every output."""
+    opt = tuple(None if t is None else t.data_ptr() for t in (slopes, sinks, gate)) + (float(softcap), float(out_scale))
     if head_dim not in DECODE_HEAD_DIMS or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
         return False
     G = num_heads // num_kv_heads
@@ -537,7 +539,7 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
               num_kv_heads, head_dim, page_size, float(scale), int(window), pages, *opt, _stream())
     if plan.cut_tokens:
         _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), plan.rows.data_ptr(), plan.cut_tokens,
-                  tile_part.data_ptr(), num_heads, head_dim, plan.cuts, opt[1], opt[2], _stream())
+                  tile_part.data_ptr(), num_heads, head_dim, plan.cuts, opt[1], opt[2], opt[4], _stream())
     return True
 
 

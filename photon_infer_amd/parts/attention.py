@@ -50,6 +50,7 @@ class PagedAttention(Mixer):
         softcap: Optional[float] = None,
         out_scale: float = 1.0,
         names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight"),
+        any_head_size: bool = False,
     ):
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
@@ -69,10 +70,12 @@ class PagedAttention(Mixer):
         self.o_size = self.num_heads * self.value_dim
         # what only the general kernels and the separate rotation serve
         self.with_options = self.value_dim != self.head_dim or self.softcap > 0.0 or self.out_scale != 1.0
-        if self.value_dim == self.head_dim:
-            ops.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
-        else:
+        if any_head_size and self.head_dim % 16:     # a head size that only the general kernels take
+            self.with_options = True
+        if self.with_options:
             ops.check_general_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim)
+        else:
+            ops.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
 
     def tensor_specs(self) -> List[TensorSpec]:
         specs = [TensorSpec(self.names[0], (self.q_size, self.hidden_size))]
