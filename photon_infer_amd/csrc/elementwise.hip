@@ -280,18 +280,18 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
 // float32.  Optionally the stream's row gets a bias added on the way (x[t, :] += xb): the bias of
 // the product that follows, which then only accumulates.
 template <typename TO, typename TI, typename TB>
-__global__ void clamped_glu_kernel(TO* __restrict__ out, const TI* __restrict__ gu, const TB* __restrict__ bg,
-                                   const TB* __restrict__ bu, float limit, float alpha, int I, float* __restrict__ x,
-                                   const TB* __restrict__ xb, int D) {
+__global__ __launch_bounds__(256) void clamped_glu_kernel(TO* __restrict__ out, const TI* __restrict__ gu, const TB* __restrict__ bg,
+                                                          const TB* __restrict__ bu, float limit, float alpha, int I, float* __restrict__ x,
+                                                          const TB* __restrict__ xb, int D) {
   const long t = blockIdx.x;
-  const TI* row = gu + t * 2 * I;
-  for (int i = threadIdx.x; i < I; i += blockDim.x) {
+  const int i = blockIdx.y * 256 + threadIdx.x;      // a thread per feature; the grid covers max(I, D)
+  if (i < I) {
+    const TI* row = gu + t * 2 * I;
     const float g = fminf(to_float(row[i]) + to_float(bg[i]), limit);
     const float u = fminf(fmaxf(to_float(row[I + i]) + to_float(bu[i]), -limit), limit);
     out[t * I + i] = from_float<TO>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
   }
-  if (x)
-    for (int i = threadIdx.x; i < D; i += blockDim.x) x[t * D + i] += to_float(xb[i]);
+  if (x && i < D) x[t * D + i] += to_float(xb[i]);
 }
 
 extern "C" int pi_clamped_glu(void* out, int out_dtype, const void* gu, int gu_dtype, const void* bg, const void* bu,
@@ -299,7 +299,9 @@ extern "C" int pi_clamped_glu(void* out, int out_dtype, const void* gu, int gu_d
                               hipStream_t stream) {
   PI_REQUIRE(T >= 0 && I > 0 && (!x || (xb && D > 0)), "clamped unit: bad sizes T=%d I=%d D=%d", T, I, D);
   if (T == 0) return 0;
-  const dim3 grid(T), block(256);
+  const int widest = x && D > I ? D : I;
+  PI_REQUIRE((widest + 255) / 256 <= 65535, "clamped unit: rows of %d features are too wide", widest);
+  const dim3 grid(T, (widest + 255) / 256), block(256);
 #define PI_GLU(TO_, TI_, TB_)                                                                                               \
   hipLaunchKernelGGL((clamped_glu_kernel<TO_, TI_, TB_>), grid, block, 0, stream, (TO_*)out, (const TI_*)gu, (const TB_*)bg, \
                      (const TB_*)bu, limit, alpha, I, x, (const TB_*)xb, D)

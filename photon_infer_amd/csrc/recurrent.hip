@@ -9,8 +9,8 @@
 
 #define PI_CONV_MAX_TAPS 8
 #define PI_CONV_SEGMENT 64
-#define PI_SCAN_COLUMNS 16      // value columns of a wave
-#define PI_SCAN_CHUNK 8         // tokens staged through LDS at a time
+#define PI_SCAN_COLUMNS 16      // value columns of a block: four walking waves of four columns each
+#define PI_SCAN_WAVES 4
 
 __device__ inline float silu_f(float v) { return v / (1.0f + expf(-v)); }
 __device__ inline float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
@@ -102,21 +102,69 @@ extern "C" int pi_causal_conv_silu(float* out, long out_stride, const float* in,
   return pi_check_launch("causal_conv_silu");
 }
 
-// ------------------------------------------------------------------ how a wave holds a state
-// A wave owns 16 value columns of one head of one request.  A column's state (one value per
-// key channel / state row) is split over four lanes: lane = 4 * column + part, and a lane keeps
-// the rows part * NR .. part * NR + NR - 1 in registers.  Rows beyond the real size are zero in
-// every staged vector, so they stay zero in the state and the walk needs no tests.
-__device__ inline float quad_sum(float v) {
-  v += __shfl_xor(v, 1, PI_WAVE);
-  v += __shfl_xor(v, 2, PI_WAVE);
+// ------------------------------------------------------------------ how a block walks a state
+// A block owns 16 value columns of one head of one request.  Four of its five waves keep the
+// state, four columns each: a column's state (one value per key channel / state row) is split
+// over the sixteen lanes of a row of the wave, lane = 16 * column + part, and a lane keeps the rows
+// part * NR .. part * NR + NR - 1 in registers; a sum over a column is four adds through the
+// data-parallel primitives (quad_perm, row_ror), no trip through LDS.  Rows beyond the real size
+// are zero in every staged vector, so they stay zero in the state and the walk needs no tests.
+// The fifth wave stages the tokens' vectors through LDS a chunk ahead of the walk, so that the
+// memory's latency lies behind it; everything of a token that does not depend on the state
+// (decays, unit vectors, beta) is made beforehand, once per token and head, by a kernel that is
+// parallel in the tokens.  The walk itself is multiply-adds on registers and LDS reads.  One
+// barrier per chunk hands a buffer over.
+//
+// In memory a request's state is kept in the walk's own order, [head][slice of four columns][i][lane]
+// (NR * 64 floats per slice), so that a wave loads and stores it in whole 256-byte rows.
+// Nothing else reads it; a cleared row is a zero state in any order.
+template <int CTRL>
+__device__ inline float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+// the sum over the 16 lanes of a row, in every lane of the row
+__device__ inline float row16_sum(float v) {
+  v += dpp_move<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x124>(v);      // row_ror 4
+  v += dpp_move<0x128>(v);      // row_ror 8
   return v;
 }
 
 static inline int scan_rows_per_lane(int rows) {
-  for (int nr = 4; nr <= 64; nr *= 2)
-    if (4 * nr >= rows) return nr;
+  for (int nr = 1; nr <= 16; nr *= 2)
+    if (16 * nr >= rows) return nr;
   return 0;
+}
+
+// Floats of one request's state for `heads` heads of `rows` x `cols` (0: rows beyond 256).
+extern "C" long pi_scan_state_floats(int heads, int rows, int cols) {
+  const int nr = scan_rows_per_lane(rows);
+  return (long)heads * ((cols + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS) * PI_SCAN_WAVES * nr * PI_WAVE;
+}
+
+template <int NR> struct ScanShape {
+  static constexpr int W = 16 * NR;                 // rows of a staged vector
+  static constexpr int CH = NR >= 16 ? 8 : 16;      // tokens per chunk
+};
+
+// `cn` tokens' vectors of `size` floats (token t at src + t * stride) into LDS rows of W floats, zeros
+// from `size` on, by one wave; `vec`: size % 4 == 0 and 16-byte accesses are allowed
+template <int W>
+__device__ inline void stage_vectors(float* dst, const float* __restrict__ src, long stride, int cn, int size, bool vec, int lane) {
+  if (vec) {
+    constexpr int Q = W / 4;
+    for (int i = lane; i < cn * Q; i += PI_WAVE) {
+      const int tt = i / Q, r = (i - tt * Q) * 4;
+      const float4 v = r < size ? *reinterpret_cast<const float4*>(src + tt * stride + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+      *reinterpret_cast<float4*>(dst + tt * W + r) = v;
+    }
+  } else {
+    for (int i = lane; i < cn * W; i += PI_WAVE) {
+      const int tt = i / W, r = i - tt * W;
+      dst[i] = r < size ? src[tt * stride + r] : 0.f;
+    }
+  }
 }
 
 // ------------------------------------------------------------------ state-space recurrence
@@ -125,63 +173,77 @@ static inline int scan_rows_per_lane(int rows) {
 //   y_t = S^T C_t + D[h] x_t
 // x, B, C are columns of the convolution's output: x at 0, B at H * P, C at H * P + G * N.
 template <int NR>
-__global__ __launch_bounds__(PI_WAVE) void state_space_scan_kernel(
+__global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void state_space_scan_kernel(
     float* __restrict__ y, long y_stride, const float* __restrict__ xbc, long xbc_stride, const float* __restrict__ dt_raw,
     long dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
     const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ state, long state_stride, int H, int P,
-    int N, int G) {
-  constexpr int W = 4 * NR;
-  __shared__ float sB[PI_SCAN_CHUNK][W], sC[PI_SCAN_CHUNK][W], sx[PI_SCAN_CHUNK][PI_SCAN_COLUMNS], sdt[PI_SCAN_CHUNK], sa[PI_SCAN_CHUNK];
-  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int col = blockIdx.z * PI_SCAN_COLUMNS + lane / 4, part = lane % 4;
+    int N, int G, int vec) {
+  constexpr int W = ScanShape<NR>::W, CH = ScanShape<NR>::CH;
+  __shared__ __attribute__((aligned(16))) float sB[2][CH * W];
+  __shared__ __attribute__((aligned(16))) float sC[2][CH * W];
+  __shared__ float sx[2][CH][PI_SCAN_COLUMNS], sdt[2][CH], sa[2][CH];
+  const int r = blockIdx.x, h = blockIdx.y, z = blockIdx.z;
+  const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE, part = lane % 16;
   const int g = h / (H / G);
   const int qs = q_start[r], n = q_start[r + 1] - qs;
   if (n <= 0) return;
-  float* S = state + (long)slots[r] * state_stride + (long)h * N * P;
-  const bool live = col < P;
-  float s[NR];
-#pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int row = part * NR + i;
-    s[i] = (live && row < N) ? S[(long)row * P + col] : 0.f;
-  }
-  const float A = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
-  const long b_col = (long)H * P + (long)g * N, c_col = b_col + (long)G * N, x_col = (long)h * P + blockIdx.z * PI_SCAN_COLUMNS;
-  for (int c0 = 0; c0 < n; c0 += PI_SCAN_CHUNK) {
-    const int cn = n - c0 < PI_SCAN_CHUNK ? n - c0 : PI_SCAN_CHUNK;
-    __syncthreads();
-    for (int i = lane; i < cn * W; i += PI_WAVE) {
-      const int tt = i / W, row = i - tt * W;
-      const float* src = xbc + (long)(qs + c0 + tt) * xbc_stride;
-      sB[tt][row] = row < N ? src[b_col + row] : 0.f;
-      sC[tt][row] = row < N ? src[c_col + row] : 0.f;
-    }
+  const int chunks = (n + CH - 1) / CH;
+  const long b_col = (long)H * P + (long)g * N, c_col = b_col + (long)G * N, x_col = (long)h * P + z * PI_SCAN_COLUMNS;
+
+  auto fill = [&](int c) {      // the staging wave
+    const int buf = c & 1, t0 = c * CH, cn = n - t0 < CH ? n - t0 : CH;
+    const float* src = xbc + (long)(qs + t0) * xbc_stride;
+    stage_vectors<W>(sB[buf], src + b_col, xbc_stride, cn, N, vec != 0, lane);
+    stage_vectors<W>(sC[buf], src + c_col, xbc_stride, cn, N, vec != 0, lane);
     for (int i = lane; i < cn * PI_SCAN_COLUMNS; i += PI_WAVE) {
       const int tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
-      sx[tt][cc] = blockIdx.z * PI_SCAN_COLUMNS + cc < P ? xbc[(long)(qs + c0 + tt) * xbc_stride + x_col + cc] : 0.f;
+      sx[buf][tt][cc] = z * PI_SCAN_COLUMNS + cc < P ? src[tt * xbc_stride + x_col + cc] : 0.f;
     }
     if (lane < cn) {
-      const float dt = softplus_f(dt_raw[(long)(qs + c0 + lane) * dt_stride + h] + bias);
-      sdt[lane] = dt;
-      sa[lane] = expf(-A * dt);
+      const float dt = softplus_f(dt_raw[(long)(qs + t0 + lane) * dt_stride + h] + dt_bias[h]);
+      sdt[buf][lane] = dt;
+      sa[buf][lane] = expf(-expf(A_log[h]) * dt);
+    }
+  };
+
+  float s[NR];
+  const int cw = wave * 4 + lane / 16;                 // this lane's column within the block
+  const int col = z * PI_SCAN_COLUMNS + cw;
+  const bool live = col < P;
+  float* Sg = state + (long)slots[r] * state_stride + (((long)h * gridDim.z + z) * PI_SCAN_WAVES + (wave & 3)) * NR * PI_WAVE + lane;
+  const float skip = Dskip[h];
+  if (wave < PI_SCAN_WAVES) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i) s[i] = Sg[i * PI_WAVE];
+  } else {
+    fill(0);
+  }
+  __syncthreads();
+  for (int c = 0; c < chunks; ++c) {
+    if (wave == PI_SCAN_WAVES) {
+      if (c + 1 < chunks) fill(c + 1);
+    } else {
+      const int buf = c & 1, cn = n - c * CH < CH ? n - c * CH : CH;
+      for (int tt = 0; tt < cn; ++tt) {
+        const float x = sx[buf][tt][cw], a = sa[buf][tt], dx = sdt[buf][tt] * x;
+        const float* Bv = &sB[buf][tt * W + part * NR];
+        const float* Cv = &sC[buf][tt * W + part * NR];
+        float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          s[i] = fmaf(a, s[i], Bv[i] * dx);
+          if (i & 1) acc1 = fmaf(s[i], Cv[i], acc1);
+          else acc0 = fmaf(s[i], Cv[i], acc0);
+        }
+        const float acc = row16_sum(acc0 + acc1);
+        if (live && part == 0) y[(long)(qs + c * CH + tt) * y_stride + (long)h * P + col] = fmaf(skip, x, acc);
+      }
     }
     __syncthreads();
-    for (int tt = 0; tt < cn; ++tt) {
-      const float x = sx[tt][lane / 4], a = sa[tt], dx = sdt[tt] * x;
-      float acc = 0.f;
-#pragma unroll
-      for (int i = 0; i < NR; ++i) {
-        s[i] = fmaf(a, s[i], sB[tt][part * NR + i] * dx);
-        acc = fmaf(s[i], sC[tt][part * NR + i], acc);
-      }
-      acc = quad_sum(acc);
-      if (live && part == 0) y[(long)(qs + c0 + tt) * y_stride + (long)h * P + col] = fmaf(skip, x, acc);
-    }
   }
+  if (wave < PI_SCAN_WAVES) {
 #pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int row = part * NR + i;
-    if (live && row < N) S[(long)row * P + col] = s[i];
+    for (int i = 0; i < NR; ++i) Sg[i * PI_WAVE] = s[i];
   }
 }
 
@@ -190,20 +252,21 @@ extern "C" int pi_state_space_scan(float* y, long y_stride, const float* xbc, lo
                                    const int* slots, int R, float* state, long state_stride, int H, int P, int N, int G,
                                    hipStream_t stream) {
   PI_REQUIRE(H > 0 && H <= 65535 && P > 0 && N > 0 && G > 0 && H % G == 0, "state space: bad sizes heads=%d vdim=%d state=%d groups=%d", H, P, N, G);
-  PI_REQUIRE(R >= 0 && state_stride >= (long)H * N * P, "state space: a state row of %ld floats cannot hold %d x %d x %d", state_stride, H, N, P);
   const int nr = scan_rows_per_lane(N);
   PI_REQUIRE(nr > 0, "state space: a state of %d rows per head is more than 256", N);
+  PI_REQUIRE(R >= 0 && state_stride >= pi_scan_state_floats(H, N, P), "state space: a state row of %ld floats cannot hold %d x %d x %d", state_stride, H, N, P);
   if (R == 0) return 0;
-  const dim3 grid(R, H, (P + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block(PI_WAVE);
+  const int vec = N % 4 == 0 && xbc_stride % 4 == 0 && ((long)H * P) % 4 == 0 && (uintptr_t)xbc % 16 == 0;
+  const dim3 grid(R, H, (P + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block((PI_SCAN_WAVES + 1) * PI_WAVE);
 #define PI_LAUNCH_SS(NR_)                                                                                                     \
   hipLaunchKernelGGL(state_space_scan_kernel<NR_>, grid, block, 0, stream, y, y_stride, xbc, xbc_stride, dt_raw, dt_stride,  \
-                     dt_bias, A_log, Dskip, q_start, slots, state, state_stride, H, P, N, G)
+                     dt_bias, A_log, Dskip, q_start, slots, state, state_stride, H, P, N, G, vec)
   switch (nr) {
+    case 1: PI_LAUNCH_SS(1); break;
+    case 2: PI_LAUNCH_SS(2); break;
     case 4: PI_LAUNCH_SS(4); break;
     case 8: PI_LAUNCH_SS(8); break;
-    case 16: PI_LAUNCH_SS(16); break;
-    case 32: PI_LAUNCH_SS(32); break;
-    default: PI_LAUNCH_SS(64); break;
+    default: PI_LAUNCH_SS(16); break;
   }
 #undef PI_LAUNCH_SS
   return pi_check_launch("state_space_scan");
@@ -254,99 +317,145 @@ extern "C" int pi_gated_group_norm(void* out, int out_dtype, long out_stride, co
 //   q^ = q / sqrt(sum q^2 + unit_eps) * q_scale;  k^ = k / sqrt(sum k^2 + unit_eps);
 //   decay[c] = exp(-exp(A_log[h]) * softplus(a[h, c] + dt_bias[h, c]));  beta = sigmoid(b[h]);
 //   S <- diag(decay) S;  u = beta * (v - S^T k^);  S <- S + k^ u^T;  o = S^T q^
-// q, k, v are columns of the convolution's output (q at 0, k at G * d, v at 2 * G * d).  A column
-// of S never meets another column, so a wave walks its 16 columns alone; unit vectors, decays and
-// beta of a chunk of tokens are made while the chunk is staged.
+// q, k, v are columns of the convolution's output (q at 0, k at G * d, v at 2 * G * d).
+//
+// First, once per token and head and in place: unit vectors over q and k, decays over a, beta over b.
+// One wave per (token, key head) and per (token, head).
+__global__ __launch_bounds__(PI_WAVE) void delta_prepare_kernel(float* __restrict__ qkv, long qkv_stride, float* __restrict__ a,
+                                                               long a_stride, const float* __restrict__ dt_bias,
+                                                               const float* __restrict__ A_log, float* __restrict__ b,
+                                                               long b_stride, int H, int G, int d, float q_scale, float unit_eps) {
+  const long t = blockIdx.x;
+  const int j = blockIdx.y, lane = threadIdx.x;
+  if (j < G) {
+    float* q = qkv + t * qkv_stride + (long)j * d;
+    float* k = q + (long)G * d;
+    float q2 = 0.f, k2 = 0.f;
+    for (int c = lane; c < d; c += PI_WAVE) {
+      q2 = fmaf(q[c], q[c], q2);
+      k2 = fmaf(k[c], k[c], k2);
+    }
+    const float qn = q_scale / sqrtf(wave_sum(q2) + unit_eps), kn = 1.0f / sqrtf(wave_sum(k2) + unit_eps);
+    for (int c = lane; c < d; c += PI_WAVE) {
+      q[c] *= qn;
+      k[c] *= kn;
+    }
+    return;
+  }
+  const int h = j - G;
+  const float A = expf(A_log[h]);
+  float* ar = a + t * a_stride + (long)h * d;
+  for (int c = lane; c < d; c += PI_WAVE) ar[c] = expf(-A * softplus_f(ar[c] + dt_bias[(long)h * d + c]));
+  if (lane == 0) b[t * b_stride + h] = sigmoid_f(b[t * b_stride + h]);
+}
+
+// Then the walk: q^, k^ and v from qkv, decays from a, beta from b.  A column of S never meets another
+// column, so a wave walks its four columns alone.
 template <int NR>
-__global__ __launch_bounds__(PI_WAVE) void delta_scan_kernel(
-    float* __restrict__ o, long o_stride, const float* __restrict__ qkv, long qkv_stride, const float* __restrict__ a,
-    long a_stride, const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ b, long b_stride,
-    const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ state, long state_stride, int H, int G,
-    int d, int dv, float q_scale, float unit_eps) {
-  constexpr int W = 4 * NR;
-  __shared__ float sq[PI_SCAN_CHUNK][W], sk[PI_SCAN_CHUNK][W], sg[PI_SCAN_CHUNK][W], sv[PI_SCAN_CHUNK][PI_SCAN_COLUMNS], sbeta[PI_SCAN_CHUNK];
-  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int col = blockIdx.z * PI_SCAN_COLUMNS + lane / 4, part = lane % 4;
+__global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kernel(
+    float* __restrict__ o, long o_stride, const float* __restrict__ qkv, long qkv_stride, const float* __restrict__ decay,
+    long decay_stride, const float* __restrict__ beta, long beta_stride, const int* __restrict__ q_start,
+    const int* __restrict__ slots, float* __restrict__ state, long state_stride, int H, int G, int d, int dv, int vec) {
+  constexpr int W = ScanShape<NR>::W, CH = ScanShape<NR>::CH;
+  __shared__ __attribute__((aligned(16))) float sq[2][CH * W];
+  __shared__ __attribute__((aligned(16))) float sk[2][CH * W];
+  __shared__ __attribute__((aligned(16))) float sg[2][CH * W];
+  __shared__ float sv[2][CH][PI_SCAN_COLUMNS], sbeta[2][CH];
+  const int r = blockIdx.x, h = blockIdx.y, z = blockIdx.z;
+  const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE, part = lane % 16;
   const int g = h / (H / G);
   const int qs = q_start[r], n = q_start[r + 1] - qs;
   if (n <= 0) return;
-  float* S = state + (long)slots[r] * state_stride + (long)h * d * dv;
-  const bool live = col < dv;
+  const int chunks = (n + CH - 1) / CH;
+  const long q_col = (long)g * d, k_col = (long)G * d + (long)g * d, v_col = 2L * G * d + (long)h * dv + z * PI_SCAN_COLUMNS;
+
+  auto fill = [&](int c) {      // the staging wave
+    const int buf = c & 1, t0 = c * CH, cn = n - t0 < CH ? n - t0 : CH;
+    const float* src = qkv + (long)(qs + t0) * qkv_stride;
+    stage_vectors<W>(sq[buf], src + q_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
+    stage_vectors<W>(sk[buf], src + k_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
+    stage_vectors<W>(sg[buf], decay + (long)(qs + t0) * decay_stride + (long)h * d, decay_stride, cn, d, (vec & 2) != 0, lane);
+    for (int i = lane; i < cn * PI_SCAN_COLUMNS; i += PI_WAVE) {
+      const int tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
+      sv[buf][tt][cc] = z * PI_SCAN_COLUMNS + cc < dv ? src[tt * qkv_stride + v_col + cc] : 0.f;
+    }
+    if (lane < cn) sbeta[buf][lane] = beta[(long)(qs + t0 + lane) * beta_stride + h];
+  };
+
   float s[NR];
+  const int cw = wave * 4 + lane / 16;                 // this lane's column within the block
+  const int col = z * PI_SCAN_COLUMNS + cw;
+  const bool live = col < dv;
+  float* Sg = state + (long)slots[r] * state_stride + (((long)h * gridDim.z + z) * PI_SCAN_WAVES + (wave & 3)) * NR * PI_WAVE + lane;
+  if (wave < PI_SCAN_WAVES) {
 #pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int row = part * NR + i;
-    s[i] = (live && row < d) ? S[(long)row * dv + col] : 0.f;
+    for (int i = 0; i < NR; ++i) s[i] = Sg[i * PI_WAVE];
+  } else {
+    fill(0);
   }
-  const float A = expf(A_log[h]);
-  const long q_col = (long)g * d, k_col = (long)G * d + (long)g * d, v_col = 2L * G * d + (long)h * dv + blockIdx.z * PI_SCAN_COLUMNS;
-  for (int c0 = 0; c0 < n; c0 += PI_SCAN_CHUNK) {
-    const int cn = n - c0 < PI_SCAN_CHUNK ? n - c0 : PI_SCAN_CHUNK;
-    __syncthreads();
-    for (int tt = 0; tt < cn; ++tt) {
-      const long t = qs + c0 + tt;
-      const float* src = qkv + t * qkv_stride;
-      float q2 = 0.f, k2 = 0.f;
-      for (int c = lane; c < d; c += PI_WAVE) {
-        const float qv = src[q_col + c], kv = src[k_col + c];
-        q2 = fmaf(qv, qv, q2);
-        k2 = fmaf(kv, kv, k2);
+  __syncthreads();
+  for (int c = 0; c < chunks; ++c) {
+    if (wave == PI_SCAN_WAVES) {
+      if (c + 1 < chunks) fill(c + 1);
+    } else {
+      const int buf = c & 1, cn = n - c * CH < CH ? n - c * CH : CH;
+      for (int tt = 0; tt < cn; ++tt) {
+        const float* qv = &sq[buf][tt * W + part * NR];
+        const float* kv = &sk[buf][tt * W + part * NR];
+        const float* gv = &sg[buf][tt * W + part * NR];
+        float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          s[i] *= gv[i];
+          if (i & 1) d1 = fmaf(s[i], kv[i], d1);
+          else d0 = fmaf(s[i], kv[i], d0);
+        }
+        const float u = sbeta[buf][tt] * (sv[buf][tt][cw] - row16_sum(d0 + d1));
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          s[i] = fmaf(kv[i], u, s[i]);
+          if (i & 1) a1 = fmaf(s[i], qv[i], a1);
+          else a0 = fmaf(s[i], qv[i], a0);
+        }
+        const float acc = row16_sum(a0 + a1);
+        if (live && part == 0) o[(long)(qs + c * CH + tt) * o_stride + (long)h * dv + col] = acc;
       }
-      const float qn = q_scale / sqrtf(wave_sum(q2) + unit_eps), kn = 1.0f / sqrtf(wave_sum(k2) + unit_eps);
-      for (int c = lane; c < W; c += PI_WAVE) {
-        const bool in = c < d;
-        sq[tt][c] = in ? src[q_col + c] * qn : 0.f;
-        sk[tt][c] = in ? src[k_col + c] * kn : 0.f;
-        sg[tt][c] = in ? expf(-A * softplus_f(a[t * a_stride + (long)h * d + c] + dt_bias[(long)h * d + c])) : 0.f;
-      }
-      if (lane < PI_SCAN_COLUMNS) sv[tt][lane] = blockIdx.z * PI_SCAN_COLUMNS + lane < dv ? src[v_col + lane] : 0.f;
-      if (lane == PI_SCAN_COLUMNS) sbeta[tt] = sigmoid_f(b[t * b_stride + h]);
     }
     __syncthreads();
-    for (int tt = 0; tt < cn; ++tt) {
-      float dot = 0.f;
-#pragma unroll
-      for (int i = 0; i < NR; ++i) {
-        s[i] *= sg[tt][part * NR + i];
-        dot = fmaf(s[i], sk[tt][part * NR + i], dot);
-      }
-      const float u = sbeta[tt] * (sv[tt][lane / 4] - quad_sum(dot));
-      float acc = 0.f;
-#pragma unroll
-      for (int i = 0; i < NR; ++i) {
-        s[i] = fmaf(sk[tt][part * NR + i], u, s[i]);
-        acc = fmaf(s[i], sq[tt][part * NR + i], acc);
-      }
-      acc = quad_sum(acc);
-      if (live && part == 0) o[(long)(qs + c0 + tt) * o_stride + (long)h * dv + col] = acc;
-    }
   }
+  if (wave < PI_SCAN_WAVES) {
 #pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int row = part * NR + i;
-    if (live && row < d) S[(long)row * dv + col] = s[i];
+    for (int i = 0; i < NR; ++i) Sg[i * PI_WAVE] = s[i];
   }
 }
 
-extern "C" int pi_delta_scan(float* o, long o_stride, const float* qkv, long qkv_stride, const float* a, long a_stride,
-                             const float* dt_bias, const float* A_log, const float* b, long b_stride, const int* q_start,
-                             const int* slots, int R, float* state, long state_stride, int H, int G, int d, int dv, float q_scale,
-                             float unit_eps, hipStream_t stream) {
-  PI_REQUIRE(H > 0 && H <= 65535 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", H, G, d, dv);
-  PI_REQUIRE(R >= 0 && state_stride >= (long)H * d * dv, "delta rule: a state row of %ld floats cannot hold %d x %d x %d", state_stride, H, d, dv);
+// qkv, a and b are changed in place (unit vectors, decays, beta); o gets the read-outs.
+extern "C" int pi_delta_scan(float* o, long o_stride, float* qkv, long qkv_stride, float* a, long a_stride,
+                             const float* dt_bias, const float* A_log, float* b, long b_stride, const int* q_start,
+                             const int* slots, int R, int T, float* state, long state_stride, int H, int G, int d, int dv,
+                             float q_scale, float unit_eps, hipStream_t stream) {
+  PI_REQUIRE(H > 0 && H <= 32767 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", H, G, d, dv);
   const int nr = scan_rows_per_lane(d);
   PI_REQUIRE(nr > 0, "delta rule: keys of %d channels are more than 256", d);
-  if (R == 0) return 0;
-  const dim3 grid(R, H, (dv + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block(PI_WAVE);
-#define PI_LAUNCH_DELTA(NR_)                                                                                                 \
-  hipLaunchKernelGGL(delta_scan_kernel<NR_>, grid, block, 0, stream, o, o_stride, qkv, qkv_stride, a, a_stride, dt_bias,    \
-                     A_log, b, b_stride, q_start, slots, state, state_stride, H, G, d, dv, q_scale, unit_eps)
+  PI_REQUIRE(R >= 0 && T >= 0 && state_stride >= pi_scan_state_floats(H, d, dv), "delta rule: a state row of %ld floats cannot hold %d x %d x %d", state_stride, H, d, dv);
+  if (R == 0 || T == 0) return 0;
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(T, G + H), dim3(PI_WAVE), 0, stream, qkv, qkv_stride, a, a_stride, dt_bias, A_log, b,
+                     b_stride, H, G, d, q_scale, unit_eps);
+  if (pi_check_launch("delta_prepare")) return -1;
+  // bit 0: q and k may be fetched 16 bytes at a time; bit 1: the decays too
+  const int vec = (d % 4 == 0 && qkv_stride % 4 == 0 && (uintptr_t)qkv % 16 == 0 ? 1 : 0) |
+                  (d % 4 == 0 && a_stride % 4 == 0 && (uintptr_t)a % 16 == 0 ? 2 : 0);
+  const dim3 grid(R, H, (dv + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block((PI_SCAN_WAVES + 1) * PI_WAVE);
+#define PI_LAUNCH_DELTA(NR_)                                                                                                   \
+  hipLaunchKernelGGL(delta_scan_kernel<NR_>, grid, block, 0, stream, o, o_stride, qkv, qkv_stride, a, a_stride, b, b_stride, \
+                     q_start, slots, state, state_stride, H, G, d, dv, vec)
   switch (nr) {
+    case 1: PI_LAUNCH_DELTA(1); break;
+    case 2: PI_LAUNCH_DELTA(2); break;
     case 4: PI_LAUNCH_DELTA(4); break;
     case 8: PI_LAUNCH_DELTA(8); break;
-    case 16: PI_LAUNCH_DELTA(16); break;
-    case 32: PI_LAUNCH_DELTA(32); break;
-    default: PI_LAUNCH_DELTA(64); break;
+    default: PI_LAUNCH_DELTA(16); break;
   }
 #undef PI_LAUNCH_DELTA
   return pi_check_launch("delta_scan");

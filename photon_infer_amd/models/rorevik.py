@@ -24,13 +24,17 @@ from ..parts.model import ModelSpec, RunEntry
 from ..registry import register_architecture
 
 
-def _mixer(cfg: RorevikConfig, m):
+def _mixer(cfg: RorevikConfig, m, ropes: dict):
     D, eps = cfg.width, cfg.norm_eps
     if isinstance(m, ParallelMixerConfig):
         a, r = m.left, m.right
         rope = None
         if a.rot_dims:
-            rope = POSITION_ENCODINGS.make("rope", head_dim=a.dim, theta=a.rot_base, interleaved=True, rotary_dim=a.rot_dims)
+            # layers that rotate alike share the part, and with it a step's table of cosines and sines
+            key = (a.dim, a.rot_dims, a.rot_base)
+            if key not in ropes:
+                ropes[key] = POSITION_ENCODINGS.make("rope", head_dim=a.dim, theta=a.rot_base, interleaved=True, rotary_dim=a.rot_dims)
+            rope = ropes[key]
         left = MIXERS.make("attention", hidden_size=D, num_heads=a.heads, num_kv_heads=a.kv_heads, head_dim=a.dim, position=rope,
                            scale=a.scale, value_dim=a.vdim, softcap=a.softcap, out_scale=m.left_scale, names=("q", "k", "v", "o"), any_head_size=True)
         right = MIXERS.make("state_space", hidden_size=D, num_heads=r.heads, value_dim=r.vdim, state_dim=r.state, groups=r.groups,
@@ -48,7 +52,7 @@ def _mixer(cfg: RorevikConfig, m):
 def build_rorevik(cfg: RorevikConfig) -> ModelSpec:
     D, eps = cfg.width, cfg.norm_eps
     norm = lambda: NORMS.make("rmsnorm", dim=D, eps=eps, tensor_name="")
-    layers, ignorable = [], []
+    layers, ignorable, ropes = [], [], {}
     for i, layer in enumerate(cfg.layers):
         norm2 = ffn = None
         if layer.mlp is not None:
@@ -56,7 +60,7 @@ def build_rorevik(cfg: RorevikConfig) -> ModelSpec:
             ffn = ("mlp.", FEED_FORWARDS.make("clamped_glu", hidden_size=D, intermediate_size=layer.mlp.ff, limit=layer.mlp.limit))
         else:
             ignorable.append(f"l{i}.norm2")      # a layer without a feed-forward has no use for its norm
-        block = BLOCKS.make("prenorm", norm1=("norm1", norm()), mixer=("mix.", _mixer(cfg, layer.mixer)), norm2=norm2, ffn=ffn)
+        block = BLOCKS.make("prenorm", norm1=("norm1", norm()), mixer=("mix.", _mixer(cfg, layer.mixer, ropes)), norm2=norm2, ffn=ffn)
         layers.append((f"l{i}.", block))
     embedding = PositionedEmbedding(cfg.vocab, D, cfg.max_positions, scale=cfg.embedding_scale, norm=("embed.norm", norm()),
                                     tensor_name="embed", position_name="pos")

@@ -796,6 +796,32 @@ def _f32_rows(t: torch.Tensor, T: int, cols: int, what: str) -> int:
     return _rows(t, what)
 
 
+SCAN_COLUMNS = 16        # value columns of a block of the state walks: four waves of four columns
+
+
+def _scan_rows_per_lane(rows: int) -> int:
+    nr = next((n for n in (1, 2, 4, 8, 16) if 16 * n >= rows), 0)
+    if nr == 0 or rows <= 0:
+        raise KernelError(f"state walk: {rows} rows per head are not within 1 .. 256")
+    return nr
+
+
+def scan_state_floats(heads: int, rows: int, cols: int) -> int:
+    """Floats of one request's state [heads, rows, cols] as the state walks keep it: in their own order,
+    [head][slice of 16 columns][wave][i][lane], where lane = 16 * column + part of wave w holds row
+    part * NR + i of column 16 * slice + 4 * w + column (NR: the rows per lane, the power of two up to 16 with
+    16 * NR >= rows), padded to whole slices and rows."""
+    return int(heads) * -(-int(cols) // SCAN_COLUMNS) * 4 * _scan_rows_per_lane(rows) * 64     # the kernels' own count: pi_scan_state_floats
+
+
+def unpack_scan_state(row: torch.Tensor, heads: int, rows: int, cols: int) -> torch.Tensor:
+    """One request's state as [heads, rows, cols], from the walks' own order (for tests and inspection)."""
+    floats, nr, slices = scan_state_floats(heads, rows, cols), _scan_rows_per_lane(rows), -(-cols // SCAN_COLUMNS)
+    t = row[:floats].view(heads, slices, 4, nr, 4, 16)               # [h, z, wave, i, column, part]
+    t = t.permute(0, 5, 3, 1, 2, 4).reshape(heads, 16 * nr, slices * SCAN_COLUMNS)   # row = part * nr + i, col = z * 16 + wave * 4 + column
+    return t[:, :rows, :cols]
+
+
 def causal_conv_silu(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], ctx,
                      state: torch.Tensor) -> None:
     """out[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - (taps - 1) + j, c]) within each request of the
@@ -822,7 +848,7 @@ def causal_conv_silu(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, b
 def state_space_scan(y: torch.Tensor, xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
                      skip: torch.Tensor, ctx, state: torch.Tensor, heads: int, value_dim: int, state_dim: int, groups: int) -> None:
     """The state-space recurrence over the step's tokens, request by request, from and into the
-    requests' state rows (``state`` float32 [slots, >= heads * state_dim * value_dim], rows ``ctx.slots``):
+    requests' state rows (``state`` float32 [slots, >= scan_state_floats(heads, state_dim, value_dim)], rows ``ctx.slots``):
     ``S <- exp(-exp(a_log) * dt') S + dt' B x^T``, ``y = S^T C + skip * x`` with ``dt' = softplus(dt + dt_bias)``.
     ``xbc`` float32 rows hold x [heads * value_dim], B and C [groups * state_dim each]; ``dt`` float32 [T, heads]
     (a column view is fine); ``y`` float32 [T, heads * value_dim]."""
@@ -833,7 +859,7 @@ def state_space_scan(y: torch.Tensor, xbc: torch.Tensor, dt: torch.Tensor, dt_bi
     ldd = _f32_rows(dt, T, heads, "state space steps")
     for t, what in ((dt_bias, "step bias"), (a_log, "decay"), (skip, "skip")):
         _f32_vector(t, heads, f"state space {what}")
-    _state_rows(state, heads * state_dim * value_dim, "state space")
+    _state_rows(state, scan_state_floats(heads, state_dim, value_dim), "state space")
     _i32(ctx.q_start, "q_start", ctx.R + 1)
     _i32(ctx.slots, "slots", ctx.R)
     _lib.call("core", "pi_state_space_scan", y.data_ptr(), ldy, xbc.data_ptr(), ldx, dt.data_ptr(), ldd, dt_bias.data_ptr(),
@@ -859,10 +885,11 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: tor
                ctx, state: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int, q_scale: float,
                unit_eps: float) -> None:
     """The gated delta rule with a decay per head and key channel over the step's tokens, from and
-    into the requests' state rows (``state`` float32 [slots, >= heads * key_dim * value_dim]):
+    into the requests' state rows (``state`` float32 [slots, >= scan_state_floats(heads, key_dim, value_dim)]):
     ``S <- diag(decay) S; u = beta (v - S^T k^); S <- S + k^ u^T; o = S^T q^`` with unit vectors
     ``k^``, ``q^`` (the latter times ``q_scale``), ``decay = exp(-exp(a_log) * softplus(a + dt_bias))``,
-    ``beta = sigmoid(b)``.  ``qkv`` float32 rows hold q and k [kv_heads * key_dim each] and v
+    ``beta = sigmoid(b)``.  ``qkv``, ``a`` and ``b`` are CHANGED IN PLACE: a first kernel turns them into the unit
+    vectors, the decays and beta, once per token and head, before the walk reads them.  ``qkv`` float32 rows hold q and k [kv_heads * key_dim each] and v
     [heads * value_dim]; ``a`` float32 [T, heads * key_dim]; ``b`` float32 [T, heads] (a column view
     is fine); ``o`` float32 [T, heads * value_dim]."""
     _gpu(o, qkv, a, dt_bias, a_log, b, state)
@@ -873,11 +900,11 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: tor
     ldb = _f32_rows(b, T, heads, "delta rule beta")
     _f32_vector(dt_bias, heads * key_dim, "delta rule decay bias")
     _f32_vector(a_log, heads, "delta rule decay rate")
-    _state_rows(state, heads * key_dim * value_dim, "delta rule")
+    _state_rows(state, scan_state_floats(heads, key_dim, value_dim), "delta rule")
     _i32(ctx.q_start, "q_start", ctx.R + 1)
     _i32(ctx.slots, "slots", ctx.R)
     _lib.call("core", "pi_delta_scan", o.data_ptr(), ldo, qkv.data_ptr(), ldq, a.data_ptr(), lda, dt_bias.data_ptr(), a_log.data_ptr(),
-              b.data_ptr(), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, state.data_ptr(), state.stride(0), heads,
+              b.data_ptr(), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, T, state.data_ptr(), state.stride(0), heads,
               kv_heads, key_dim, value_dim, float(q_scale), float(unit_eps), _stream())
 
 

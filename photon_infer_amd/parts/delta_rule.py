@@ -64,7 +64,7 @@ class ChannelDeltaRule(Mixer):
                 TensorSpec("o", (D, self.v_size))]
 
     def cache_spec(self):
-        return StateSpec((self.conv_floats + self.num_heads * self.key_dim * self.value_dim,), torch.float32)
+        return StateSpec((self.conv_floats + ops.scan_state_floats(self.num_heads, self.key_dim, self.value_dim),), torch.float32)
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)

@@ -52,7 +52,7 @@ class StateSpaceMixer(Mixer):
                 TensorSpec("D", (H,), "bias"), TensorSpec("norm", (self.inner,), "norm"), TensorSpec("o", (D, self.inner))]
 
     def cache_spec(self):
-        return StateSpec((self.conv_floats + self.num_heads * self.state_dim * self.value_dim,), torch.float32)
+        return StateSpec((self.conv_floats + ops.scan_state_floats(self.num_heads, self.state_dim, self.value_dim),), torch.float32)
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)

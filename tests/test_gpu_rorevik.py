@@ -103,19 +103,20 @@ def test_state_space_recurrence_whole_in_portions_and_token_by_token(sizes):
         want[n] = P.state_space_recurrence(x, B, C, P.softplus(dt + dt_bias), A_log, D)
     slot = {"a": 3, "b": 1}
     for cuts in ({"a": [83], "b": [10]}, {"a": [1], "b": [1]}, {"a": [2, 17, 1, 40], "b": [3, 2]}, {"a": [9], "b": [10]}):
-        state = torch.zeros((4, H * N * Pd + 3), device=DEV)
+        floats = ops.scan_state_floats(H, N, Pd)
+        state = torch.zeros((4, floats + 3), device=DEV)
         got = {n: [] for n in T}
         for step in in_steps(T, cuts):
             xbc = dev32(torch.cat([data[n][0][i:j] for n, i, j in step]))
             dt = dev32(torch.cat([data[n][1][i:j] for n, i, j in step]))
             y = torch.empty((xbc.shape[0], H * Pd), device=DEV)
             ops.state_space_scan(y, xbc, dt, dev32(dt_bias), dev32(A_log), dev32(D), state_ctx([j - i for _, i, j in step], [slot[n] for n, _, _ in step]),
-                                 state[:, :H * N * Pd], H, Pd, N, G)
+                                 state[:, :floats], H, Pd, N, G)
             for (n, i, j), part in zip(step, torch.split(y, [j - i for _, i, j in step])):
                 got[n].append(part)
         for n in T:
             close(torch.cat(got[n]), want[n][0].reshape(T[n], -1), f"{sizes} {n} cut {cuts[n]}", 5e-5)
-            close(state[slot[n], :H * N * Pd].view(H, N, Pd), want[n][1], f"{sizes} {n} state after {cuts[n]}", 5e-5)
+            close(ops.unpack_scan_state(state[slot[n]], H, N, Pd), want[n][1], f"{sizes} {n} state after {cuts[n]}", 5e-5)
         assert bool((state[0] == 0).all()) and bool((state[2] == 0).all())
 
 
@@ -140,7 +141,7 @@ def test_delta_rule_whole_in_portions_and_token_by_token(sizes):
     want = {n: delta_plain(*data[n], dt_bias, A_log, H, d) for n in T}
     slot = {"a": 0, "b": 2}
     for cuts in ({"a": [90], "b": [11]}, {"a": [1], "b": [1]}, {"a": [2, 30, 1, 8, 9], "b": [4, 1]}, {"a": [7], "b": [11]}):
-        state = torch.zeros((3, H * d * dv), device=DEV)
+        state = torch.zeros((3, ops.scan_state_floats(H, d, dv)), device=DEV)
         got = {n: [] for n in T}
         for step in in_steps(T, cuts):
             cat = lambda idx: torch.cat([data[n][idx][i:j].reshape(j - i, -1) for n, i, j in step])
@@ -152,7 +153,7 @@ def test_delta_rule_whole_in_portions_and_token_by_token(sizes):
                 got[n].append(part)
         for n in T:
             close(torch.cat(got[n]), want[n][0].reshape(T[n], -1), f"{sizes} {n} cut {cuts[n]}", 5e-5)
-            close(state[slot[n]].view(H, d, dv), want[n][1], f"{sizes} {n} state after {cuts[n]}", 5e-5)
+            close(ops.unpack_scan_state(state[slot[n]], H, d, dv), want[n][1], f"{sizes} {n} state after {cuts[n]}", 5e-5)
         assert bool((state[1] == 0).all())
 
 
@@ -177,7 +178,7 @@ def test_a_write_is_recalled_after_hundreds_of_tokens_and_forgotten_by_its_chann
         a = torch.full((T, H, d), -big, dtype=F64)
         a[300:300 + halvings, :, 0] = math.log(math.e ** math.log(2.0) - 1.0)    # softplus = ln 2: decay one half
         a = a.view(T, H * d)
-        state = torch.zeros((2, H * d * dv), device=DEV)
+        state = torch.zeros((2, ops.scan_state_floats(H, d, dv)), device=DEV)
         sizes = [T - 40] + [1] * 40 if decode else [64, 2, 200, 1, 3]
         outs, i, kk = [], 0, 0
         while i < T:

@@ -80,8 +80,9 @@ def test_tensor_list_and_cache_plan():
     assert len(plan.groups) == 1 and plan.groups[0].window is None
     assert plan.groups[0].owners == ((0, 0), (2, 0), (4, 0))
     shapes = {key: s.shape for key, s in plan.states}
-    ssm = ((3 - 1) * 80 + 2 * 16 * 24,)
-    delta = ((2 - 1) * (32 + 32 + 96) + 4 * 16 * 24,)
+    # the convolution's inputs, then S in the walks' order: [head][slice of 16 columns][4 waves][rows per lane][64 lanes]
+    ssm = ((3 - 1) * 80 + 2 * 2 * 4 * 1 * 64,)
+    delta = ((2 - 1) * (32 + 32 + 96) + 4 * 2 * 4 * 1 * 64,)
     assert shapes == {(0, 1): ssm, (2, 1): ssm, (4, 1): ssm, (1, 0): delta, (3, 0): delta, (5, 0): delta}
     assert all(isinstance(s, StateSpec) and s.dtype == torch.float32 for _, s in plan.states)
     # a model of delta-rule layers only keeps no pages
