@@ -143,42 +143,62 @@ extern "C" long pi_scan_state_floats(int heads, int rows, int cols) {
   return (long)heads * ((cols + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS) * PI_SCAN_WAVES * nr * PI_WAVE;
 }
 
-template <int NR> struct ScanShape {
-  static constexpr int W = 16 * NR;                 // rows of a staged vector
-  static constexpr int CH = NR >= 16 ? 8 : 16;      // tokens per chunk
+// SHORT: a step in which no request brings more than two tokens (decoding) is staged two tokens at a time:
+// few registers and little LDS, so that many blocks share a compute unit while they wait for their states.
+template <int NR, bool SHORT> struct ScanShape {
+  static constexpr int W = 16 * NR;                                   // rows of a staged vector
+  static constexpr int CH = SHORT ? 2 : (NR >= 16 ? 8 : 16);          // tokens per chunk
 };
 
-// `cn` tokens' vectors of `size` floats (token t at src + t * stride) into LDS rows of W floats, zeros
-// from `size` on, by one wave; `vec`: size % 4 == 0 and 16-byte accesses are allowed
-template <int W>
-__device__ inline void stage_vectors(float* dst, const float* __restrict__ src, long stride, int cn, int size, bool vec, int lane) {
-  if (vec) {
-    constexpr int Q = W / 4;
-    for (int i = lane; i < cn * Q; i += PI_WAVE) {
-      const int tt = i / Q, r = (i - tt * Q) * 4;
-      const float4 v = r < size ? *reinterpret_cast<const float4*>(src + tt * stride + r) : make_float4(0.f, 0.f, 0.f, 0.f);
-      *reinterpret_cast<float4*>(dst + tt * W + r) = v;
-    }
-  } else {
-    for (int i = lane; i < cn * W; i += PI_WAVE) {
-      const int tt = i / W, r = i - tt * W;
-      dst[i] = r < size ? src[tt * stride + r] : 0.f;
+// `cn` tokens' vectors of `size` floats (token t at src + t * stride) on their way into LDS rows of W floats,
+// zeros from `size` on, by one wave.  Fetching and storing are two steps, so that a chunk's fetches are all
+// in flight before the first of them is waited for.  `vec`: size % 4 == 0 and 16-byte accesses are allowed;
+// otherwise the vectors are copied one float at a time by store().
+template <int W, int CH>
+struct StagedVectors {
+  static constexpr int Q = W / 4, IT = (CH * Q + PI_WAVE - 1) / PI_WAVE;
+  float4 v[IT];
+  const float* src;
+  long stride;
+  int cn, size;
+  bool vec;
+  __device__ inline void fetch(const float* __restrict__ from, long row_stride, int tokens, int floats, bool wide, int lane) {
+    src = from; stride = row_stride; cn = tokens; size = floats; vec = wide;
+    if (!vec) return;
+#pragma unroll
+    for (int j = 0; j < IT; ++j) {
+      const int i = lane + j * PI_WAVE, tt = i / Q, r = (i - tt * Q) * 4;
+      v[j] = (tt < cn && r < size) ? *reinterpret_cast<const float4*>(src + tt * stride + r) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   }
-}
+  __device__ inline void store(float* dst, int lane) const {
+    if (vec) {
+#pragma unroll
+      for (int j = 0; j < IT; ++j) {
+        const int i = lane + j * PI_WAVE, tt = i / Q, r = (i - tt * Q) * 4;
+        if (tt < cn) *reinterpret_cast<float4*>(dst + tt * W + r) = v[j];
+      }
+    } else {
+      for (int i = lane; i < cn * W; i += PI_WAVE) {
+        const int tt = i / W, r = i - tt * W;
+        dst[i] = r < size ? src[tt * stride + r] : 0.f;
+      }
+    }
+  }
+};
 
 // ------------------------------------------------------------------ state-space recurrence
 // Per head h with group g = h / (H / G), state S [N, P] (float32, zero at the start):
 //   dt = softplus(dt_raw + dt_bias[h]);  S <- exp(-exp(A_log[h]) * dt) S + dt * B_t x_t^T;
 //   y_t = S^T C_t + D[h] x_t
 // x, B, C are columns of the convolution's output: x at 0, B at H * P, C at H * P + G * N.
-template <int NR>
+template <int NR, bool SHORT>
 __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void state_space_scan_kernel(
     float* __restrict__ y, long y_stride, const float* __restrict__ xbc, long xbc_stride, const float* __restrict__ dt_raw,
     long dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
     const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ state, long state_stride, int H, int P,
     int N, int G, int vec) {
-  constexpr int W = ScanShape<NR>::W, CH = ScanShape<NR>::CH;
+  constexpr int W = ScanShape<NR, SHORT>::W, CH = ScanShape<NR, SHORT>::CH;
   __shared__ __attribute__((aligned(16))) float sB[2][CH * W];
   __shared__ __attribute__((aligned(16))) float sC[2][CH * W];
   __shared__ float sx[2][CH][PI_SCAN_COLUMNS], sdt[2][CH], sa[2][CH];
@@ -193,14 +213,26 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void state_space_sca
   auto fill = [&](int c) {      // the staging wave
     const int buf = c & 1, t0 = c * CH, cn = n - t0 < CH ? n - t0 : CH;
     const float* src = xbc + (long)(qs + t0) * xbc_stride;
-    stage_vectors<W>(sB[buf], src + b_col, xbc_stride, cn, N, vec != 0, lane);
-    stage_vectors<W>(sC[buf], src + c_col, xbc_stride, cn, N, vec != 0, lane);
-    for (int i = lane; i < cn * PI_SCAN_COLUMNS; i += PI_WAVE) {
-      const int tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
-      sx[buf][tt][cc] = z * PI_SCAN_COLUMNS + cc < P ? src[tt * xbc_stride + x_col + cc] : 0.f;
+    StagedVectors<W, CH> Bs, Cs;
+    Bs.fetch(src + b_col, xbc_stride, cn, N, vec != 0, lane);
+    Cs.fetch(src + c_col, xbc_stride, cn, N, vec != 0, lane);
+    constexpr int XI = (CH * PI_SCAN_COLUMNS + PI_WAVE - 1) / PI_WAVE;
+    float xs[XI];
+#pragma unroll
+    for (int j = 0; j < XI; ++j) {
+      const int i = lane + j * PI_WAVE, tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
+      xs[j] = (tt < cn && z * PI_SCAN_COLUMNS + cc < P) ? src[tt * xbc_stride + x_col + cc] : 0.f;
+    }
+    const float raw = lane < cn ? dt_raw[(long)(qs + t0 + lane) * dt_stride + h] : 0.f;
+    Bs.store(sB[buf], lane);
+    Cs.store(sC[buf], lane);
+#pragma unroll
+    for (int j = 0; j < XI; ++j) {
+      const int i = lane + j * PI_WAVE;
+      if (i < CH * PI_SCAN_COLUMNS) (&sx[buf][0][0])[i] = xs[j];
     }
     if (lane < cn) {
-      const float dt = softplus_f(dt_raw[(long)(qs + t0 + lane) * dt_stride + h] + dt_bias[h]);
+      const float dt = softplus_f(raw + dt_bias[h]);
       sdt[buf][lane] = dt;
       sa[buf][lane] = expf(-expf(A_log[h]) * dt);
     }
@@ -224,6 +256,7 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void state_space_sca
       if (c + 1 < chunks) fill(c + 1);
     } else {
       const int buf = c & 1, cn = n - c * CH < CH ? n - c * CH : CH;
+#pragma unroll 2
       for (int tt = 0; tt < cn; ++tt) {
         const float x = sx[buf][tt][cw], a = sa[buf][tt], dx = sdt[buf][tt] * x;
         const float* Bv = &sB[buf][tt * W + part * NR];
@@ -249,7 +282,7 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void state_space_sca
 
 extern "C" int pi_state_space_scan(float* y, long y_stride, const float* xbc, long xbc_stride, const float* dt_raw, long dt_stride,
                                    const float* dt_bias, const float* A_log, const float* Dskip, const int* q_start,
-                                   const int* slots, int R, float* state, long state_stride, int H, int P, int N, int G,
+                                   const int* slots, int R, int longest, float* state, long state_stride, int H, int P, int N, int G,
                                    hipStream_t stream) {
   PI_REQUIRE(H > 0 && H <= 65535 && P > 0 && N > 0 && G > 0 && H % G == 0, "state space: bad sizes heads=%d vdim=%d state=%d groups=%d", H, P, N, G);
   const int nr = scan_rows_per_lane(N);
@@ -258,9 +291,10 @@ extern "C" int pi_state_space_scan(float* y, long y_stride, const float* xbc, lo
   if (R == 0) return 0;
   const int vec = N % 4 == 0 && xbc_stride % 4 == 0 && ((long)H * P) % 4 == 0 && (uintptr_t)xbc % 16 == 0;
   const dim3 grid(R, H, (P + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block((PI_SCAN_WAVES + 1) * PI_WAVE);
-#define PI_LAUNCH_SS(NR_)                                                                                                     \
-  hipLaunchKernelGGL(state_space_scan_kernel<NR_>, grid, block, 0, stream, y, y_stride, xbc, xbc_stride, dt_raw, dt_stride,  \
+#define PI_LAUNCH_SS1(NR_, SHORT_)                                                                                                       \
+  hipLaunchKernelGGL((state_space_scan_kernel<NR_, SHORT_>), grid, block, 0, stream, y, y_stride, xbc, xbc_stride, dt_raw, dt_stride, \
                      dt_bias, A_log, Dskip, q_start, slots, state, state_stride, H, P, N, G, vec)
+#define PI_LAUNCH_SS(NR_) do { if (longest <= 2) PI_LAUNCH_SS1(NR_, true); else PI_LAUNCH_SS1(NR_, false); } while (0)
   switch (nr) {
     case 1: PI_LAUNCH_SS(1); break;
     case 2: PI_LAUNCH_SS(2); break;
@@ -269,6 +303,7 @@ extern "C" int pi_state_space_scan(float* y, long y_stride, const float* xbc, lo
     default: PI_LAUNCH_SS(16); break;
   }
 #undef PI_LAUNCH_SS
+#undef PI_LAUNCH_SS1
   return pi_check_launch("state_space_scan");
 }
 
@@ -351,12 +386,12 @@ __global__ __launch_bounds__(PI_WAVE) void delta_prepare_kernel(float* __restric
 
 // Then the walk: q^, k^ and v from qkv, decays from a, beta from b.  A column of S never meets another
 // column, so a wave walks its four columns alone.
-template <int NR>
+template <int NR, bool SHORT>
 __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kernel(
     float* __restrict__ o, long o_stride, const float* __restrict__ qkv, long qkv_stride, const float* __restrict__ decay,
     long decay_stride, const float* __restrict__ beta, long beta_stride, const int* __restrict__ q_start,
     const int* __restrict__ slots, float* __restrict__ state, long state_stride, int H, int G, int d, int dv, int vec) {
-  constexpr int W = ScanShape<NR>::W, CH = ScanShape<NR>::CH;
+  constexpr int W = ScanShape<NR, SHORT>::W, CH = ScanShape<NR, SHORT>::CH;
   __shared__ __attribute__((aligned(16))) float sq[2][CH * W];
   __shared__ __attribute__((aligned(16))) float sk[2][CH * W];
   __shared__ __attribute__((aligned(16))) float sg[2][CH * W];
@@ -372,14 +407,27 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
   auto fill = [&](int c) {      // the staging wave
     const int buf = c & 1, t0 = c * CH, cn = n - t0 < CH ? n - t0 : CH;
     const float* src = qkv + (long)(qs + t0) * qkv_stride;
-    stage_vectors<W>(sq[buf], src + q_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
-    stage_vectors<W>(sk[buf], src + k_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
-    stage_vectors<W>(sg[buf], decay + (long)(qs + t0) * decay_stride + (long)h * d, decay_stride, cn, d, (vec & 2) != 0, lane);
-    for (int i = lane; i < cn * PI_SCAN_COLUMNS; i += PI_WAVE) {
-      const int tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
-      sv[buf][tt][cc] = z * PI_SCAN_COLUMNS + cc < dv ? src[tt * qkv_stride + v_col + cc] : 0.f;
+    StagedVectors<W, CH> qs_, ks_, gs_;
+    qs_.fetch(src + q_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
+    ks_.fetch(src + k_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
+    gs_.fetch(decay + (long)(qs + t0) * decay_stride + (long)h * d, decay_stride, cn, d, (vec & 2) != 0, lane);
+    constexpr int XI = (CH * PI_SCAN_COLUMNS + PI_WAVE - 1) / PI_WAVE;
+    float vs[XI];
+#pragma unroll
+    for (int j = 0; j < XI; ++j) {
+      const int i = lane + j * PI_WAVE, tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
+      vs[j] = (tt < cn && z * PI_SCAN_COLUMNS + cc < dv) ? src[tt * qkv_stride + v_col + cc] : 0.f;
     }
-    if (lane < cn) sbeta[buf][lane] = beta[(long)(qs + t0 + lane) * beta_stride + h];
+    const float bt = lane < cn ? beta[(long)(qs + t0 + lane) * beta_stride + h] : 0.f;
+    qs_.store(sq[buf], lane);
+    ks_.store(sk[buf], lane);
+    gs_.store(sg[buf], lane);
+#pragma unroll
+    for (int j = 0; j < XI; ++j) {
+      const int i = lane + j * PI_WAVE;
+      if (i < CH * PI_SCAN_COLUMNS) (&sv[buf][0][0])[i] = vs[j];
+    }
+    if (lane < CH) sbeta[buf][lane] = bt;
   };
 
   float s[NR];
@@ -399,6 +447,7 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
       if (c + 1 < chunks) fill(c + 1);
     } else {
       const int buf = c & 1, cn = n - c * CH < CH ? n - c * CH : CH;
+#pragma unroll 2
       for (int tt = 0; tt < cn; ++tt) {
         const float* qv = &sq[buf][tt * W + part * NR];
         const float* kv = &sk[buf][tt * W + part * NR];
@@ -433,7 +482,7 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
 // qkv, a and b are changed in place (unit vectors, decays, beta); o gets the read-outs.
 extern "C" int pi_delta_scan(float* o, long o_stride, float* qkv, long qkv_stride, float* a, long a_stride,
                              const float* dt_bias, const float* A_log, float* b, long b_stride, const int* q_start,
-                             const int* slots, int R, int T, float* state, long state_stride, int H, int G, int d, int dv,
+                             const int* slots, int R, int T, int longest, float* state, long state_stride, int H, int G, int d, int dv,
                              float q_scale, float unit_eps, hipStream_t stream) {
   PI_REQUIRE(H > 0 && H <= 32767 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", H, G, d, dv);
   const int nr = scan_rows_per_lane(d);
@@ -447,9 +496,10 @@ extern "C" int pi_delta_scan(float* o, long o_stride, float* qkv, long qkv_strid
   const int vec = (d % 4 == 0 && qkv_stride % 4 == 0 && (uintptr_t)qkv % 16 == 0 ? 1 : 0) |
                   (d % 4 == 0 && a_stride % 4 == 0 && (uintptr_t)a % 16 == 0 ? 2 : 0);
   const dim3 grid(R, H, (dv + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block((PI_SCAN_WAVES + 1) * PI_WAVE);
-#define PI_LAUNCH_DELTA(NR_)                                                                                                   \
-  hipLaunchKernelGGL(delta_scan_kernel<NR_>, grid, block, 0, stream, o, o_stride, qkv, qkv_stride, a, a_stride, b, b_stride, \
+#define PI_LAUNCH_DELTA1(NR_, SHORT_)                                                                                                   \
+  hipLaunchKernelGGL((delta_scan_kernel<NR_, SHORT_>), grid, block, 0, stream, o, o_stride, qkv, qkv_stride, a, a_stride, b, b_stride, \
                      q_start, slots, state, state_stride, H, G, d, dv, vec)
+#define PI_LAUNCH_DELTA(NR_) do { if (longest <= 2) PI_LAUNCH_DELTA1(NR_, true); else PI_LAUNCH_DELTA1(NR_, false); } while (0)
   switch (nr) {
     case 1: PI_LAUNCH_DELTA(1); break;
     case 2: PI_LAUNCH_DELTA(2); break;
@@ -458,5 +508,6 @@ extern "C" int pi_delta_scan(float* o, long o_stride, float* qkv, long qkv_strid
     default: PI_LAUNCH_DELTA(16); break;
   }
 #undef PI_LAUNCH_DELTA
+#undef PI_LAUNCH_DELTA1
   return pi_check_launch("delta_scan");
 }

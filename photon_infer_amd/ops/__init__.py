@@ -863,8 +863,8 @@ def state_space_scan(y: torch.Tensor, xbc: torch.Tensor, dt: torch.Tensor, dt_bi
     _i32(ctx.q_start, "q_start", ctx.R + 1)
     _i32(ctx.slots, "slots", ctx.R)
     _lib.call("core", "pi_state_space_scan", y.data_ptr(), ldy, xbc.data_ptr(), ldx, dt.data_ptr(), ldd, dt_bias.data_ptr(),
-              a_log.data_ptr(), skip.data_ptr(), ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, state.data_ptr(),
-              state.stride(0), heads, value_dim, state_dim, groups, _stream())
+              a_log.data_ptr(), skip.data_ptr(), ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R,
+              int(getattr(ctx, "max_q_len", 0) or T), state.data_ptr(), state.stride(0), heads, value_dim, state_dim, groups, _stream())
 
 
 def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, parts: int,
@@ -904,7 +904,7 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: tor
     _i32(ctx.q_start, "q_start", ctx.R + 1)
     _i32(ctx.slots, "slots", ctx.R)
     _lib.call("core", "pi_delta_scan", o.data_ptr(), ldo, qkv.data_ptr(), ldq, a.data_ptr(), lda, dt_bias.data_ptr(), a_log.data_ptr(),
-              b.data_ptr(), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, T, state.data_ptr(), state.stride(0), heads,
+              b.data_ptr(), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, T, int(getattr(ctx, "max_q_len", 0) or T), state.data_ptr(), state.stride(0), heads,
               kv_heads, key_dim, value_dim, float(q_scale), float(unit_eps), _stream())
 
 

@@ -19,9 +19,9 @@ _SIGNATURES = {
         "pi_embedding_positions": [P, P, P, I, P, P, F, I, I, I, I, P],
         "pi_clamped_glu": [P, I, P, I, P, P, P, I, F, F, I, I, P, I, P],
         "pi_causal_conv_silu": [P, L, P, L, P, P, I, I, I, P, P, I, I, P, L, P],
-        "pi_state_space_scan": [P, L, P, L, P, L, P, P, P, P, P, I, P, L, I, I, I, I, P],
+        "pi_state_space_scan": [P, L, P, L, P, L, P, P, P, P, P, I, I, P, L, I, I, I, I, P],
         "pi_gated_group_norm": [P, I, L, P, L, P, L, P, F, F, I, I, I, P],
-        "pi_delta_scan": [P, L, P, L, P, L, P, P, P, L, P, P, I, I, P, L, I, I, I, I, F, F, P],
+        "pi_delta_scan": [P, L, P, L, P, L, P, P, P, L, P, P, I, I, I, P, L, I, I, I, I, F, F, P],
         "pi_rmsnorm": [P, I, P, P, P, I, F, I, I, P, I, L, P],
         "pi_swiglu": [P, P, I, I, I, I, P],
         "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, I, P],
