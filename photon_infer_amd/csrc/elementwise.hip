@@ -282,29 +282,33 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
 template <typename TO, typename TI, typename TB>
 __global__ __launch_bounds__(256) void clamped_glu_kernel(TO* __restrict__ out, const TI* __restrict__ gu, const TB* __restrict__ bg,
                                                           const TB* __restrict__ bu, float limit, float alpha, int I, float* __restrict__ x,
-                                                          const TB* __restrict__ xb, int D) {
+                                                          const TB* __restrict__ xb, int D, int block) {
   const long t = blockIdx.x;
   const int i = blockIdx.y * 256 + threadIdx.x;      // a thread per feature; the grid covers max(I, D)
   if (i < I) {
     const TI* row = gu + t * 2 * I;
-    const float g = fminf(to_float(row[i]) + to_float(bg[i]), limit);
-    const float u = fminf(fmaxf(to_float(row[I + i]) + to_float(bu[i]), -limit), limit);
+    // block == 0: [gate | up] in halves, biases bg and bu; block == b: gate and up interleaved in blocks of b
+    // columns, and so are the biases, all in bg
+    const int gc = block ? (i / block) * 2 * block + i % block : i, uc = block ? gc + block : I + i;
+    const float g = fminf(to_float(row[gc]) + to_float(block ? bg[gc] : bg[i]), limit);
+    const float u = fminf(fmaxf(to_float(row[uc]) + to_float(block ? bg[uc] : bu[i]), -limit), limit);
     out[t * I + i] = from_float<TO>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
   }
   if (x && i < D) x[t * D + i] += to_float(xb[i]);
 }
 
 extern "C" int pi_clamped_glu(void* out, int out_dtype, const void* gu, int gu_dtype, const void* bg, const void* bu,
-                              const void* xb, int b_dtype, float limit, float alpha, int T, int I, float* x, int D,
+                              const void* xb, int b_dtype, float limit, float alpha, int T, int I, float* x, int D, int interleave,
                               hipStream_t stream) {
-  PI_REQUIRE(T >= 0 && I > 0 && (!x || (xb && D > 0)), "clamped unit: bad sizes T=%d I=%d D=%d", T, I, D);
+  PI_REQUIRE(interleave >= 0 && (interleave == 0 || I % interleave == 0), "clamped unit: interleave block %d does not divide %d", interleave, I);
+  PI_REQUIRE(T >= 0 && I >= 0 && (!x || (xb && D > 0)), "clamped unit: bad sizes T=%d I=%d D=%d", T, I, D);
   if (T == 0) return 0;
   const int widest = x && D > I ? D : I;
   PI_REQUIRE((widest + 255) / 256 <= 65535, "clamped unit: rows of %d features are too wide", widest);
   const dim3 grid(T, (widest + 255) / 256), block(256);
 #define PI_GLU(TO_, TI_, TB_)                                                                                               \
   hipLaunchKernelGGL((clamped_glu_kernel<TO_, TI_, TB_>), grid, block, 0, stream, (TO_*)out, (const TI_*)gu, (const TB_*)bg, \
-                     (const TB_*)bu, limit, alpha, I, x, (const TB_*)xb, D)
+                     (const TB_*)bu, limit, alpha, I, x, (const TB_*)xb, D, interleave)
   if (out_dtype == PI_F32 && gu_dtype == PI_F32 && b_dtype == PI_F32) PI_GLU(float, float, float);
   else if (out_dtype == PI_BF16 && gu_dtype == PI_F32 && b_dtype == PI_BF16) PI_GLU(bf16_t, float, bf16_t);
   else if (out_dtype == PI_BF16 && gu_dtype == PI_BF16 && b_dtype == PI_BF16) PI_GLU(bf16_t, bf16_t, bf16_t);

@@ -30,7 +30,24 @@ PI_DEFINE_MODULE(bf16)
 #define BK 64
 #define TILE_ELEMS (BM * BK)                // a tile's slab in LDS: rows of 128 bytes
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3, EPI_CLAMPED_GLU = 4 };
+
+// the gated epilogues store one output column per pair of input columns, in bfloat16
+#define EPI_GATED(E) ((E) == EPI_SWIGLU || (E) == EPI_CLAMPED_GLU)
+
+// What the clamped gated unit needs beside the products: biases in the order of W's rows (gate and up
+// interleaved by 16), the clamp and the sigmoid's factor.
+struct GluArgs {
+  const float* bias;
+  float limit, alpha;
+};
+
+// g' = min(g + bg, limit), u' = clamp(u + bu, -limit, limit): g' * sigmoid(alpha * g') * (u' + 1)
+__device__ inline float clamped_glu_mul(float g, float u, float bg, float bu, float limit, float alpha) {
+  g = fminf(g + bg, limit);
+  u = fminf(fmaxf(u + bu, -limit), limit);
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * alpha * g)) * (u + 1.0f);
+}
 
 // silu(g) * u for a bfloat16 result: the hardware exponential and reciprocal (1 ulp each) are
 // far inside the rounding of the store
@@ -51,7 +68,8 @@ __device__ inline uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits
 
 template <int EPI>
 __device__ inline void store_rows32(float* patch, const f32x16_t& acc0, const f32x16_t& acc1, void* C, int ld, int row0,
-                                    int rows_left, int cols_left, int lane, bool wide) {
+                                    int rows_left, int cols_left, int lane, bool wide, GluArgs glu = GluArgs{nullptr, 0.f, 0.f},
+                                    long col0 = 0) {
   const int half = lane / 32, ccol = lane % 32;
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
@@ -63,7 +81,7 @@ __device__ inline void store_rows32(float* patch, const f32x16_t& acc0, const f3
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  if (EPI == EPI_SWIGLU) {
+  if (EPI_GATED(EPI)) {
     // columns 0..15 of a tile are gate rows of W, 16..31 the up rows of the same features
     bf16_t* out = reinterpret_cast<bf16_t*>(C);
 #pragma unroll
@@ -75,8 +93,17 @@ __device__ inline void store_rows32(float* patch, const f32x16_t& acc0, const f3
       const f32x4_t g0 = *reinterpret_cast<const f32x4_t*>(g), g1 = *reinterpret_cast<const f32x4_t*>(g + 4);
       const f32x4_t u0 = *reinterpret_cast<const f32x4_t*>(g + 16), u1 = *reinterpret_cast<const f32x4_t*>(g + 20);
       float o[8];
+      if (EPI == EPI_CLAMPED_GLU) {
+        const float* bg = glu.bias + col0 + j * 32 + q * 8;      // col0: the corner's first input column
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { o[e] = silu_mul(g0[e], u0[e]); o[4 + e] = silu_mul(g1[e], u1[e]); }
+        for (int e = 0; e < 4; ++e) {
+          o[e] = clamped_glu_mul(g0[e], u0[e], bg[e], bg[16 + e], glu.limit, glu.alpha);
+          o[4 + e] = clamped_glu_mul(g1[e], u1[e], bg[4 + e], bg[20 + e], glu.limit, glu.alpha);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { o[e] = silu_mul(g0[e], u0[e]); o[4 + e] = silu_mul(g1[e], u1[e]); }
+      }
       bf16_t* dst = out + (row0 + r) * ld + oc;
       if (wide && j * 32 + 16 + q * 8 + 8 <= cols_left) {
         *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
@@ -145,7 +172,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
                                                         const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
                                                         int tiles_n, int k_per_split, const int* __restrict__ group_of_tile,
                                                         const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
-                                                        long group_stride) {
+                                                        long group_stride, GluArgs glu) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   constexpr int ROW = BK;                   // rows of 128 bytes, no padding (see the large-tile kernel)
   constexpr int TILE = BM * ROW;
@@ -185,7 +212,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     M = tile_rows[t];
     A += r0 * lda;
     W += (long)grp * group_stride;
-    Cv = reinterpret_cast<char*>(Cv) + r0 * ldc * (EPI == EPI_BF16 || EPI == EPI_SWIGLU ? 2 : 4);
+    Cv = reinterpret_cast<char*>(Cv) + r0 * ldc * (EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4);
   }
   const long m0 = (long)tile_m * BM, n0 = (long)tile_n * BN;
 
@@ -302,11 +329,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     const long mw = m0 + wm * 64, nw = n0 + wn * 64;
     const int rows_left = (int)min((long)64, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
     float* patch = reinterpret_cast<float*>(lds) + wave * PATCH_FLOATS;
-    const int esize = EPI == EPI_BF16 || EPI == EPI_SWIGLU ? 2 : 4;
-    char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI == EPI_SWIGLU ? nw / 2 : nw)) * esize;
+    const int esize = EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4;
+    char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI_GATED(EPI) ? nw / 2 : nw)) * esize;
     const bool wide = (ldc * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(corner) % 16 == 0;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) store_rows32<EPI>(patch, acc[i][0], acc[i][1], corner, (int)ldc, i * 32, rows_left, cols_left, lane, wide);
+    for (int i = 0; i < 2; ++i) store_rows32<EPI>(patch, acc[i][0], acc[i][1], corner, (int)ldc, i * 32, rows_left, cols_left, lane, wide, glu, nw);
   }
 }
 
@@ -330,7 +357,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
 template <int EPI>
 __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
                                                             const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
-                                                            int tiles_n, int k_per_split) {
+                                                            int tiles_n, int k_per_split, GluArgs glu) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   constexpr int ROW = BK;                       // rows of 128 bytes, no padding: the loads write LDS themselves, lane after lane
   constexpr int TILE = GM * ROW;
@@ -457,11 +484,11 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
     const long mw = m0 + wm * 128, nw = n0 + wn * 64;
     const int rows_left = (int)min((long)128, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
     float* patch = reinterpret_cast<float*>(lds) + wave * PATCH_FLOATS;
-    const int esize = EPI == EPI_BF16 || EPI == EPI_SWIGLU ? 2 : 4;
-    char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI == EPI_SWIGLU ? nw / 2 : nw)) * esize;
+    const int esize = EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4;
+    char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI_GATED(EPI) ? nw / 2 : nw)) * esize;
     const bool wide = (ldc * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(corner) % 16 == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) store_rows32<EPI>(patch, acc[i][0], acc[i][1], corner, (int)ldc, i * 32, rows_left, cols_left, lane, wide);
+    for (int i = 0; i < 4; ++i) store_rows32<EPI>(patch, acc[i][0], acc[i][1], corner, (int)ldc, i * 32, rows_left, cols_left, lane, wide, glu, nw);
   }
 }
 
@@ -482,7 +509,7 @@ static const size_t kLdsBytes = 4 * TILE_ELEMS * sizeof(uint16_t);   // 65,536 b
 
 template <int EPI>
 static int launch(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K, int splits,
-                  hipStream_t stream) {
+                  hipStream_t stream, GluArgs glu = GluArgs{nullptr, 0.f, 0.f}) {
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_kernel<EPI>),
@@ -503,13 +530,13 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
       big_configured = true;
     }
     hipLaunchKernelGGL((gemm_mfma_big_kernel<EPI>), dim3((unsigned)big_tiles, splits), dim3(512), kBigLdsBytes, stream, C, ldc,
-                       (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, ceil_div(N, GN), kps);
+                       (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, ceil_div(N, GN), kps, glu);
     return pi_check_launch("gemm_mfma_big");
   }
   const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
   hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles_m * tiles_n, splits), dim3(256), kLdsBytes, stream, C, ldc,
                      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, tiles_n, kps, (const int*)nullptr, (const int*)nullptr,
-                     (const int*)nullptr, 0L);
+                     (const int*)nullptr, 0L, glu);
   return pi_check_launch("gemm_mfma");
 }
 
@@ -533,7 +560,7 @@ static int launch_grouped(void* C, long ldc, const void* A, long lda, const void
   const int tiles_n = ceil_div(N, BN);
   hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles * tiles_n, 1), dim3(256), kLdsBytes, stream, C, ldc,
                      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, BM, N, K, tiles_n, K, group_of_tile, tile_row0, tile_rows,
-                     group_stride);
+                     group_stride, GluArgs{nullptr, 0.f, 0.f});
   return pi_check_launch("gemm_mfma_grouped");
 }
 
@@ -584,4 +611,18 @@ extern "C" int pi_gemm_mfma(void* C, int epilogue, long ldc, const void* A, long
     case EPI_SWIGLU: return launch<EPI_SWIGLU>(C, ldc, A, lda, W, ldw, M, N, K, splits, stream);
   }
   return pi_fail("gemm_mfma: unknown epilogue %d", epilogue);
+}
+
+// C[M, N / 2] (bfloat16) = the clamped gated unit of A . W^T: W's rows and `bias` (float32 [N]) hold gate and up
+// interleaved by 16; g' = min(g + bg, limit), u' = clamp(u + bu, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1).
+extern "C" int pi_gemm_mfma_clamped_glu(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K,
+                                        const float* bias, float limit, float alpha, hipStream_t stream) {
+  PI_REQUIRE(M > 0 && N > 0 && K > 0 && bias, "gemm_mfma: bad sizes M=%d N=%d K=%d", M, N, K);
+  PI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_mfma: K (%d) and row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
+  PI_REQUIRE(256 * lda < (1L << 29) && 256 * ldw < (1L << 29), "gemm_mfma: row strides (%ld, %ld) are too long for 32-bit offsets inside a tile", lda, ldw);
+  PI_REQUIRE(ldc > 0 && ldc < (1L << 23), "gemm_mfma: the result's row stride (%ld) is too long for 32-bit offsets inside a tile", ldc);
+  PI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mfma: operands must be 16-byte aligned");
+  PI_REQUIRE(N % 32 == 0, "gemm_mfma: the gated epilogue needs N (%d) to be a multiple of 32", N);
+  PI_REQUIRE((long)ceil_div(M, BM) * ceil_div(N, BN) < 2147483647L, "gemm_mfma: too many tiles");
+  return launch<EPI_CLAMPED_GLU>(C, ldc, A, lda, W, ldw, M, N, K, 1, stream, GluArgs{bias, limit, alpha});
 }

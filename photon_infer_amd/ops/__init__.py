@@ -908,18 +908,21 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: tor
               kv_heads, key_dim, value_dim, float(q_scale), float(unit_eps), _stream())
 
 
-def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, gate_bias: torch.Tensor, up_bias: torch.Tensor, limit: float,
-                alpha: float, x: Optional[torch.Tensor] = None, x_bias: Optional[torch.Tensor] = None) -> None:
+def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, gate_bias: torch.Tensor, up_bias: Optional[torch.Tensor], limit: float,
+                alpha: float, x: Optional[torch.Tensor] = None, x_bias: Optional[torch.Tensor] = None, block: int = 0) -> None:
     """out = g * sigmoid(alpha * g) * (u + 1) with g = min(gate + gate_bias, limit) and
-    u = clamp(up + up_bias, -limit, limit); ``gate_up`` [T, 2I] holds the two products in halves.
-    With ``x`` (the float32 stream) and ``x_bias``: x[t, :] += x_bias as well, the bias of the product
-    that follows."""
+    u = clamp(up + up_bias, -limit, limit).  ``block`` = 0: ``gate_up`` [T, 2I] holds the two products in halves;
+    ``block`` = b: gate and up interleaved in blocks of b columns, and ``gate_bias`` [2I] holds both biases in the
+    same order (``up_bias`` None).  With ``x`` (the float32 stream) and ``x_bias``: x[t, :] += x_bias as well, the
+    bias of the product that follows."""
     _gpu(out, gate_up, gate_bias, up_bias, x, x_bias)
     T, I = out.shape
     if gate_up.shape != (T, 2 * I) or not (out.is_contiguous() and gate_up.is_contiguous()):
         raise KernelError(f"clamped unit: expected contiguous gate_up [{T}, {2 * I}], got {tuple(gate_up.shape)}")
-    biases = [gate_bias, up_bias] + ([x_bias] if x is not None else [])
-    if any(b.dtype != gate_bias.dtype or not b.is_contiguous() for b in biases) or gate_bias.numel() != I or up_bias.numel() != I:
+    if block < 0 or (block and (I % block or up_bias is not None or gate_bias.numel() != 2 * I)):
+        raise KernelError(f"clamped unit: interleave block {block} needs {I} % block == 0 and one bias vector of {2 * I}")
+    biases = [gate_bias] + ([up_bias] if not block else []) + ([x_bias] if x is not None else [])
+    if any(b is None or b.dtype != gate_bias.dtype or not b.is_contiguous() for b in biases) or (not block and (gate_bias.numel() != I or up_bias.numel() != I)):
         raise KernelError(f"clamped unit: biases must be contiguous [{I}] of one type")
     D = 0
     if x is not None:
@@ -927,5 +930,48 @@ def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, gate_bias: torch.Tenso
         if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[0] != T or x_bias is None or x_bias.numel() != D:
             raise KernelError(f"clamped unit: the stream must be contiguous float32 [{T}, D] with a bias [D]")
     _lib.call("core", "pi_clamped_glu", out.data_ptr(), _dt(out), gate_up.data_ptr(), _dt(gate_up), gate_bias.data_ptr(),
-              up_bias.data_ptr(), _ptr(x_bias) if x is not None else None, _dt(gate_bias), float(limit), float(alpha), T, I,
-              _ptr(x), D, _stream())
+              _ptr(up_bias), _ptr(x_bias) if x is not None else None, _dt(gate_bias), float(limit), float(alpha), T, I,
+              _ptr(x), D, int(block), _stream())
+
+
+def add_row_bias(x: torch.Tensor, bias: torch.Tensor) -> None:
+    """x[t, :] += bias (the float32 stream; the bias in float32)."""
+    _gpu(x, bias)
+    T, D = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or bias.dtype != torch.float32 or not bias.is_contiguous() or bias.numel() != D:
+        raise KernelError(f"row bias: expected a contiguous float32 stream [{T}, {D}] and a float32 bias [{D}]")
+    _lib.call("core", "pi_clamped_glu", None, PI_F32, None, PI_F32, None, None, bias.data_ptr(), PI_F32, 0.0, 0.0, T, 0,
+              x.data_ptr(), D, 0, _stream())
+
+
+def gemm_clamped_glu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, bias: torch.Tensor, limit: float, alpha: float,
+                     block: int, ws: Optional[KernelWorkspace] = None, x: Optional[torch.Tensor] = None,
+                     x_bias: Optional[torch.Tensor] = None) -> None:
+    """out[M, I] = the clamped gated unit (``clamped_glu``) of a @ w_gate_up^T + bias, where ``w_gate_up`` [2I, K] and
+    ``bias`` (float32 [2I]) hold gate and up rows in halves (``block`` 0) or interleaved in blocks of ``block``.  With
+    bfloat16 operands, blocks of 16 and more rows than the weight-streaming products take, product and unit are
+    one kernel; otherwise the product's float32 result goes through the unit's own kernel.  ``x`` and ``x_bias``
+    (float32): the stream's rows get ``x_bias`` added on the way (the bias of the product that follows), by the unit's
+    kernel where it runs, by a kernel of its own otherwise; an update of ``x`` that is pending in ``ws`` is applied first."""
+    _gpu(out, a, w_gate_up, bias)
+    if x is not None:
+        materialize(x, ws)
+    M, I = out.shape
+    if w_gate_up.shape[0] != 2 * I or a.shape != (M, w_gate_up.shape[1]) or bias.dtype != torch.float32 or bias.numel() != 2 * I:
+        raise KernelError(f"gemm_clamped_glu: shapes do not agree: a {tuple(a.shape)}, w {tuple(w_gate_up.shape)}, out {tuple(out.shape)}")
+    if M == 0:
+        return
+    if _FAST and block == 16 and a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out.is_contiguous() and bias.is_contiguous():
+        from . import fast
+        if fast.gemm_clamped_glu(out, a, w_gate_up, bias, limit, alpha, M, 2 * I, a.shape[1], _rows(a, "gemm a"), _rows(w_gate_up, "gemm w")):
+            if ws is not None:
+                ws.counts["gated_epilogues"] += 1
+            if x is not None:
+                add_row_bias(x, x_bias)
+            return
+    gu = torch.empty((M, 2 * I), dtype=torch.float32, device=a.device)
+    gemm(gu, a, w_gate_up, ws=ws)
+    if block:
+        clamped_glu(out, gu, bias, None, limit, alpha, x, x_bias, block=block)
+    else:
+        clamped_glu(out, gu, bias[:I], bias[I:], limit, alpha, x, x_bias)

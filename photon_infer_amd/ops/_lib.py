@@ -17,7 +17,7 @@ _SIGNATURES = {
     "core": {
         "pi_embedding": [P, P, I, P, I, I, I, P],
         "pi_embedding_positions": [P, P, P, I, P, P, F, I, I, I, I, P],
-        "pi_clamped_glu": [P, I, P, I, P, P, P, I, F, F, I, I, P, I, P],
+        "pi_clamped_glu": [P, I, P, I, P, P, P, I, F, F, I, I, P, I, I, P],
         "pi_causal_conv_silu": [P, L, P, L, P, P, I, I, I, P, P, I, I, P, L, P],
         "pi_state_space_scan": [P, L, P, L, P, L, P, P, P, P, P, I, I, P, L, I, I, I, I, P],
         "pi_gated_group_norm": [P, I, L, P, L, P, L, P, F, F, I, I, I, P],
@@ -45,6 +45,7 @@ _SIGNATURES = {
     "bf16": {
         "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, I, P],
         "pi_gemm_mfma_pieces": [I, I],
+        "pi_gemm_mfma_clamped_glu": [P, L, P, L, P, L, I, I, I, P, F, F, P],
         "pi_gemm_mfma_grouped": [P, I, L, P, L, P, L, L, P, P, P, I, I, I, P],
         "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, I, P],
         "pi_splitk_reduce": [P, I, L, P, I, I, I, P],

@@ -292,6 +292,17 @@ def gemm_swiglu(out, a, w, M, N, K, lda, ldw, ws: Optional[KernelWorkspace] = No
     return True
 
 
+def gemm_clamped_glu(out, a, w, bias, limit, alpha, M, N, K, lda, ldw) -> bool:
+    """``w`` [N = 2I, K] and ``bias`` (float32 [N]) with gate / up rows interleaved in blocks of 16; out [M, I]
+    bfloat16 gets the clamped gated unit of the products.  The tile kernels only: steps of more rows than the
+    weight-streaming kernels take."""
+    if not _gemm_ok(a, w, K, lda, ldw) or N % 32 or out.dtype != torch.bfloat16 or M <= SKINNY_MAX_ROWS:
+        return False
+    _lib.call("bf16", "pi_gemm_mfma_clamped_glu", out.data_ptr(), out.stride(0), a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
+              bias.data_ptr(), float(limit), float(alpha), _stream())
+    return True
+
+
 # ----------------------------------------------------------------------------- attention
 def attention_tile_rows(num_heads: int, num_kv_heads: int, head_dim: int) -> int:
     return _lib.load("bf16").pi_attention_tile_rows(num_heads, num_kv_heads, head_dim)

@@ -104,22 +104,31 @@ class ClampedGLU(FeedForward):
         g, u, d = self.names
         wg, wu = tensors[g], tensors[u]
         common = torch.float32 if torch.float32 in (wg.dtype, wu.dtype) else wg.dtype
-        self.w_gate_up = torch.cat([wg.to(common), wu.to(common)], dim=0).contiguous()       # rows [gate | up]
-        self.w_down = tensors[d]
+        wg, wu, I = wg.to(common), wu.to(common), self.intermediate_size
         f32 = lambda t: t.to(torch.float32).contiguous()
-        self.b_gate, self.b_up, self.b_down = f32(tensors[g + self.bias_suffix]), f32(tensors[u + self.bias_suffix]), f32(tensors[d + self.bias_suffix])
+        bg, bu = f32(tensors[g + self.bias_suffix]), f32(tensors[u + self.bias_suffix])
+        if common == torch.bfloat16 and I % INTERLEAVE == 0:
+            # one projection for gate and up, rows (and biases) interleaved in blocks of 16: the matrix-core kernels
+            # then hold a feature's gate and up value in the same lane and apply the unit before anything is stored
+            self.interleave = INTERLEAVE
+            pair = lambda a, b: torch.stack([a.view(I // INTERLEAVE, INTERLEAVE, -1), b.view(I // INTERLEAVE, INTERLEAVE, -1)], dim=1)
+            self.w_gate_up = pair(wg, wu).reshape(2 * I, -1).contiguous()
+            self.b_gate_up = pair(bg, bu).reshape(2 * I).contiguous()
+        else:
+            self.interleave = 0                      # rows [gate | up]
+            self.w_gate_up = torch.cat([wg, wu], dim=0).contiguous()
+            self.b_gate_up = torch.cat([bg, bu]).contiguous()
+        self.w_down, self.b_down = tensors[d], f32(tensors[d + self.bias_suffix])
 
     def streamed_weights(self) -> List[torch.Tensor]:
         return [self.w_gate_up, self.w_down]
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
-        T, I = h.shape[0], self.intermediate_size
         ws = ctx.workspace if ctx is not None else None
-        gu = torch.empty((T, 2 * I), dtype=torch.float32, device=h.device)
-        ops.gemm(gu, h, self.w_gate_up, ws=ws)
-        act = torch.empty((T, I), dtype=self.dtype, device=h.device)
-        ops.materialize(x, ws)          # the bias is added to the stream itself
-        ops.clamped_glu(act, gu, self.b_gate, self.b_up, self.limit, self.alpha, x, self.b_down)
+        act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
+        # the down projection's bias is added to the stream itself on the way, so that the product only accumulates
+        ops.gemm_clamped_glu(act, h, self.w_gate_up, self.b_gate_up, self.limit, self.alpha, self.interleave, ws=ws,
+                             x=x, x_bias=self.b_down)
         ops.gemm(x, act, self.w_down, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
 
 

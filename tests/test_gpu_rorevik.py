@@ -225,6 +225,38 @@ def test_clamped_unit_with_biases_and_the_stream_bias(dtype):
     close(xs, x + bd, "stream bias")
 
 
+@pytest.mark.parametrize("M,I,K", [(200, 96, 128), (129, 512, 320), (5, 96, 128), (300, 40, 64)])
+def test_product_and_clamped_unit_in_one_kernel(M, I, K):
+    """The gate | up product with the clamped unit as its epilogue (bfloat16, rows interleaved by 16, more rows than
+    the weight-streaming products take) against the product and the unit's own kernel, and against plain arithmetic."""
+    from photon_infer_amd import ops
+    limit, alpha = 1.2, 1.702
+    a = randn(M, K, seed=1).to(torch.bfloat16)
+    wg, wu = randn(I, K, seed=2, scale=0.3).to(torch.bfloat16), randn(I, K, seed=3, scale=0.3).to(torch.bfloat16)
+    bg, bu = randn(I, seed=4), randn(I, seed=5)
+    g = torch.clamp(a.double() @ wg.double().T + bg, max=limit)
+    u = torch.clamp(a.double() @ wu.double().T + bu, min=-limit, max=limit)
+    want = g * torch.sigmoid(alpha * g) * (u + 1.0)
+    if I % 16 == 0:
+        pair = lambda x, y: torch.stack([x.view(I // 16, 16, -1), y.view(I // 16, 16, -1)], dim=1)
+        w, b, block = pair(wg, wu).reshape(2 * I, K).contiguous(), pair(bg, bu).reshape(2 * I).contiguous(), 16
+    else:
+        w, b, block = torch.cat([wg, wu]).contiguous(), torch.cat([bg, bu]).contiguous(), 0
+    ws = ops.KernelWorkspace(torch.device(DEV))
+    ws.prepare(True)
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_clamped_glu(out, a.to(DEV), w.to(DEV), dev32(b), limit, alpha, block, ws=ws)
+    assert ws.counts["gated_epilogues"] == (1 if (block and M > 128) else 0)
+    close(out, want, f"clamped unit behind a product of {M} rows", 1e-2)
+    prev = ops.use_fast_kernels(False)
+    try:
+        slow = torch.empty_like(out)
+        ops.gemm_clamped_glu(slow, a.to(DEV), w.to(DEV), dev32(b), limit, alpha, block)
+    finally:
+        ops.use_fast_kernels(prev)
+    close(slow, want, "the same on the general kernels", 1e-2)
+
+
 def test_embedding_scaled_with_learned_positions():
     from photon_infer_amd import ops
     V, D, Pn = 50, 36, 20
@@ -543,6 +575,8 @@ def test_kernels_chosen_at_real_widths_against_the_general_kernels(tmp_path):
             for k in range(3):
                 got.append(r.step([StepEntry("a", [8 + k], [0]), StepEntry("b", [prompts["b"][60 + k]], [0]), StepEntry("c", [9 + k], [0])]))
             outs.append(torch.cat(got).float().cpu())
+            if fast:
+                assert r.workspace.counts["gated_epilogues"] > 0, dict(r.workspace.counts)
         finally:
             ops.use_fast_kernels(prev)
     err = float((outs[0] - outs[1]).abs().max())
