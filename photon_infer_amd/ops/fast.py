@@ -217,7 +217,7 @@ def ranges_product_ok(tokens: int, head_dim: int, weight_bytes: int = 0) -> bool
 def merge_ranges(out: torch.Tensor, kr: KeyRanges) -> None:
     """The merged attention output, bfloat16 [tokens, heads * head_dim], by the merging kernel."""
     _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), kr.rows.data_ptr(), kr.tokens,
-              kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count, None, None, _stream())
+              kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count, None, None, 1.0, _stream())
 
 
 def gemm_from_ranges(out, kr: KeyRanges, w, accumulate, N, ldw, ldc, may_defer, ws: Optional[KernelWorkspace]) -> bool:
