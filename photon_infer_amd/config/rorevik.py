@@ -33,7 +33,7 @@ class SoftcapAttentionConfig:
         rot = r.mapping("rot")
         cfg = cls(heads=r.integer("heads"), kv_heads=r.integer("kv_heads"), dim=r.integer("dim"), vdim=r.integer("vdim"),
                   scale=r.number("scale"), softcap=r.number("softcap") if r.has("softcap") else None,
-                  rot_dims=rot.integer("dims") if rot is not None else 0,
+                  rot_dims=rot.integer("dims", minimum=0) if rot is not None else 0,
                   rot_base=rot.number("base") if rot is not None else 1.0)
         if cfg.heads % cfg.kv_heads:
             raise ConfigError(f"{r.where}: heads ({cfg.heads}) must be a multiple of kv_heads ({cfg.kv_heads})")
